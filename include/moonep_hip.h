@@ -1,0 +1,166 @@
+/*
+ * libmoonep_hip -- C ABI of the MI355X (gfx950) MoonEP per-rank hot path.
+ *
+ * The reference has no C FFI on this path: its boundary is one Python
+ * launcher per kernel (launch_planning, launch_dispatch, ...), each of which
+ * JIT-compiles a CuTe-DSL kernel and launches it on the current stream.
+ * Every function below replaces one of those launchers; the cited
+ * reference lines are the launcher (host side) and the kernel it starts.
+ *
+ * Conventions
+ *  - plain pointers to DEVICE memory unless a parameter says "host";
+ *    sizes and strides are in the unit named by the parameter;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *    every call only enqueues work: no host synchronisation, no allocation,
+ *    safe to record into a HIP graph;
+ *  - return value: 0 = ok, negative = MEP_ERR_* (bad argument, nothing was
+ *    launched), positive = the hipError_t of a failed launch;
+ *    never throws, never exits;
+ *  - the R expert-parallel ranks' buffers are addressed as base + rank *
+ *    stride, so the same entry points serve one GPU emulating R ranks in
+ *    local HBM and a symmetric heap of peer-mapped memory;
+ *  - re-entrant for distinct buffers; calls that share output buffers must be
+ *    ordered by the caller (same stream or events).
+ */
+#ifndef MOONEP_HIP_H
+#define MOONEP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MEP_OK 0
+#define MEP_ERR_INVALID_ARG (-1)   /* null pointer, non-positive size, rank out of range */
+#define MEP_ERR_UNSUPPORTED (-2)   /* shape outside what the kernels handle        */
+#define MEP_ERR_SCRATCH (-3)       /* scratch buffer missing or too small           */
+#define MEP_ERR_ALIGNMENT (-4)     /* pointer/stride not 16-byte aligned            */
+
+/* dispatch flags */
+#define MEP_DISPATCH_WRITE_DUPS 1u /* also copy rows of negative (duplicate) entries */
+#define MEP_DISPATCH_NO_ZERO_FILL 2u
+
+/* combine modes */
+#define MEP_COMBINE_PRIMARIES 0 /* sum non-negative entries only (reference kernel)      */
+#define MEP_COMBINE_ALL 1       /* sum all K entries, one rounding                         */
+#define MEP_COMBINE_TWO_LEVEL 2 /* per-destination group sum -> bf16 -> sum (= reference
+                                   prologue + combine, without modifying the shards)       */
+
+int mep_version(void);
+const char* mep_strerror(int code);
+
+/* Bytes of device scratch mep_plan / mep_plan_ranks need for `nranks` ranks
+ * planned in one call (0 when the planner tables fit in LDS). */
+size_t mep_plan_scratch_bytes(int S, int K, int E, int R, int nranks);
+
+/*
+ * Online redundant-expert planner for one rank.
+ * Replaces launch_planning (reference moonep/planning.py:1258-1280) and
+ * PlanningKernel (reference moonep/planning.py:328-1101); results equal the
+ * reference oracle (reference tests/planning_reference.py:25-311) bit for bit.
+ *   tpe_RE          [R,E]  tokens every source rank routes to every expert
+ *   topk_SK         [S,K]  this rank's expert ids
+ *   dst             [S*K]  out: dest_rank*NvS + slot; later entries of a token
+ *                          on the same dest rank are stored as -(value)-1
+ *   cu_seqlens      [2*epn] out: padded end offset of each group on `rank`
+ *   experts_to_copy [R,epn] out: remote experts every rank hosts (-1 = free)
+ *   zero_fill       [2*epn,2] out: (first padding row, padding rows) per group
+ *   remote_stats    [2]    out: (#experts I host for others' homes... i.e.
+ *                          remote experts on me, #slots elsewhere holding mine)
+ * The src_info provenance scratch of the reference (planning.py:1036-1041)
+ * is not produced; mep_build_dedup derives the duplicate groups from dst.
+ */
+int mep_plan(const int32_t* tpe_RE, const int32_t* topk_SK, int rank, int S, int K, int E,
+             int R, int token_padding, int NvS, int32_t* dst, int32_t* cu_seqlens,
+             int32_t* experts_to_copy, int32_t* zero_fill, int32_t* remote_stats,
+             void* scratch, size_t scratch_bytes, void* stream);
+
+/*
+ * The same planner for ranks rank0 .. rank0+nranks-1 in one launch (one GPU
+ * standing in for several ranks).  topk is [nranks,S,K]; dst, cu_seqlens,
+ * zero_fill and remote_stats gain a leading [nranks] dimension;
+ * experts_to_copy stays [R,epn].
+ */
+int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int nranks, int S,
+                   int K, int E, int R, int token_padding, int NvS, int32_t* dst,
+                   int32_t* cu_seqlens, int32_t* experts_to_copy, int32_t* zero_fill,
+                   int32_t* remote_stats, void* scratch, size_t scratch_bytes, void* stream);
+
+/*
+ * Fused permute, source side.  Replaces launch_dispatch (reference
+ * moonep/dispatch.py:838-983; kernel :268-692, rows :394-433, zero-fill
+ * :467-497).  Copies hidden[s] to shards[drank][loff] for every non-negative
+ * dst entry (all entries with MEP_DISPATCH_WRITE_DUPS), scatters w[s,k] to
+ * wslots[drank][loff] for every entry, zero-fills rank's padding rows.
+ *   hidden_SH [S,H] bf16;  w_SK [S,K] fp32 or NULL;
+ *   shards: row r of rank d at shards + (d*shard_stride_rows + r)*H;
+ *   wslots: slot r of rank d at wslots + d*wslot_stride + r  (NULL iff w_SK NULL)
+ */
+int mep_dispatch(const void* hidden_SH, const float* w_SK, const int32_t* dst,
+                 const int32_t* zero_fill, void* shards, int64_t shard_stride_rows, float* wslots,
+                 int64_t wslot_stride, int rank, int S, int H, int K, int R, int epn, int NvS,
+                 int token_padding, unsigned flags, void* stream);
+
+/*
+ * Destination-side duplicate groups of `rank` from all ranks' dst.
+ * Replaces the dedup builder warps of DispatchKernel (reference
+ * moonep/dispatch.py:502-681).  Output order is deterministic (source rank,
+ * token) -- the reference's own order is not stable and its tests compare
+ * sets.  dst_RN [R, S*K]; dup_groups [NvS,3]; dup_loffs [NvS]; dup_counts [2].
+ * scratch: at least mep_dedup_scratch_bytes(S, R) bytes.
+ */
+size_t mep_dedup_scratch_bytes(int S, int R);
+int mep_build_dedup(const int32_t* dst_RN, int rank, int S, int K, int R, int NvS,
+                    int32_t* dup_groups, int32_t* dup_loffs, int32_t* dup_counts, void* scratch,
+                    size_t scratch_bytes, void* stream);
+
+/* primary row -> its duplicate rows, in place on one rank's shard.
+ * Replaces launch_dispatch_epilogue (reference moonep/dispatch_epilogue.py:366-415). */
+int mep_dispatch_epilogue(void* shard_NvS_H, const int32_t* dup_groups, const int32_t* dup_loffs,
+                          const int32_t* dup_counts, int NvS, int H, void* stream);
+
+/* fp32 sum of primary + duplicates -> bf16 -> primary row, in place.
+ * Replaces launch_combine_prologue (reference moonep/combine_prologue.py:544-599). */
+int mep_combine_prologue(void* shard_NvS_H, const int32_t* dup_groups, const int32_t* dup_loffs,
+                         const int32_t* dup_counts, int NvS, int H, void* stream);
+
+/*
+ * Top-k unpermute + K-sum + weight gather.  Replaces launch_combine
+ * (reference moonep/combine.py:565-654; kernel :210-511).  Unweighted fp32
+ * accumulation from +0.0 in ascending k, one round-to-nearest-even to bf16.
+ *   out_SH [S,H] bf16; out_SK [S,K] fp32 or NULL (then wslots may be NULL)
+ */
+int mep_combine(const void* shards, int64_t shard_stride_rows, const float* wslots,
+                int64_t wslot_stride, const int32_t* dst, void* out_SH, float* out_SK, int S,
+                int H, int K, int R, int NvS, int mode, void* stream);
+
+/*
+ * Owner-push expert-weight prefetch for `ntensors` (3 or 6) tensors in one
+ * launch.  Replaces launch_prefetch (reference moonep/prefetch.py:632-738;
+ * kernel :227-470).  For every (d,b) with experts_to_copy[d,b] owned by
+ * `rank`: pool_t[d][b] = local_t[expert - rank*epn], bytes copied verbatim.
+ *   local, pool, rank_stride_bytes, bytes_per_expert: HOST arrays of length
+ *   ntensors; pool_t slot (d,b) at pool[t] + d*rank_stride_bytes[t] +
+ *   b*bytes_per_expert[t]; bytes_per_expert % 16 == 0.
+ */
+int mep_prefetch(int ntensors, const void* const* local, void* const* pool,
+                 const int64_t* rank_stride_bytes, const int64_t* bytes_per_expert,
+                 const int32_t* experts_to_copy, int rank, int epn, int R, void* stream);
+
+/*
+ * fp32 slot reduction.  Replaces launch_grad_reduce (reference
+ * moonep/grad_reduce.py:437-543; kernel :151-389).  local_grad[le] +=
+ * reduce[src][b] over the slots holding expert rank*epn+le in (src,b)
+ * ascending order; then reduce[rank][b] = 0 for every b with
+ * experts_to_copy[rank,b] >= 0.  elems_per_expert % 4 == 0.
+ */
+int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t rank_stride_elems,
+                    const int32_t* experts_to_copy, int rank, int epn, int R,
+                    int64_t elems_per_expert, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOONEP_HIP_H */

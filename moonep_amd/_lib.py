@@ -1,0 +1,87 @@
+"""ctypes binding of libmoonep_hip.so (the C ABI declared in include/moonep_hip.h).
+
+The library is loaded on first use.  There is no fallback: if it has not been
+built, every operator raises.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmoonep_hip.so")
+
+_lock = threading.Lock()
+_lib = None
+
+# combine modes / dispatch flags (include/moonep_hip.h)
+COMBINE_PRIMARIES = 0
+COMBINE_ALL = 1
+COMBINE_TWO_LEVEL = 2
+DISPATCH_WRITE_DUPS = 1
+DISPATCH_NO_ZERO_FILL = 2
+
+_p = C.c_void_p
+_i = C.c_int
+_i64 = C.c_int64
+_sz = C.c_size_t
+
+_SIGNATURES = {
+    "mep_version": (_i, []),
+    "mep_strerror": (C.c_char_p, [_i]),
+    "mep_plan_scratch_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "mep_plan": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "mep_plan_ranks": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "mep_dispatch": (_i, [_p, _p, _p, _p, _p, _i64, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _i,
+                          C.c_uint, _p]),
+    "mep_dedup_scratch_bytes": (_sz, [_i, _i]),
+    "mep_build_dedup": (_i, [_p, _i, _i, _i, _i, _i, _p, _p, _p, _p, _sz, _p]),
+    "mep_dispatch_epilogue": (_i, [_p, _p, _p, _p, _i, _i, _p]),
+    "mep_combine_prologue": (_i, [_p, _p, _p, _p, _i, _i, _p]),
+    "mep_combine": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "mep_prefetch": (_i, [_i, C.POINTER(_p), C.POINTER(_p), C.POINTER(_i64), C.POINTER(_i64),
+                          _p, _i, _i, _i, _p]),
+    "mep_grad_reduce": (_i, [_p, _p, _i64, _p, _i, _i, _i, _i64, _p]),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+
+def lib():
+    """The loaded library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise RuntimeError(
+                        f"{LIB_PATH} is missing: build it with `python -m moonep_amd.build` "
+                        "(hipcc, gfx950). moonep_amd has no CPU or eager fallback."
+                    )
+                handle = C.CDLL(LIB_PATH)
+                for name, (res, args) in _SIGNATURES.items():
+                    fn = getattr(handle, name)
+                    fn.restype = res
+                    fn.argtypes = args
+                _lib = handle
+    return _lib
+
+
+def check(code: int, what: str) -> None:
+    """Turn a non-zero return code of the C ABI into RuntimeError."""
+    if code != 0:
+        msg = lib().mep_strerror(code).decode()
+        raise RuntimeError(f"{what} failed: {msg} (code {code})")
+
+
+def ptr(t) -> int | None:
+    """Device address of a tensor (None stays NULL)."""
+    return None if t is None else t.data_ptr()
+
+
+def current_stream() -> int:
+    import torch
+
+    return torch.cuda.current_stream().cuda_stream

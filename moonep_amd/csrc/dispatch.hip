@@ -1,0 +1,386 @@
+// Dispatch side of the hot path for gfx950: fused permute (one wave per token
+// row, the row is read once into registers and streamed to every destination
+// slot), weight scatter, padding zero-fill, duplicate-group builder and the
+// destination-side duplicate expansion.
+#include "mep_common.h"
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = kWavesPerBlock * MEP_WAVE;
+
+struct DispatchArgs {
+  const uint16_t* hidden;  // [S,H] bf16
+  const float* w;          // [S,K] or null
+  const int* dst;          // [S*K]
+  const int* zero_fill;    // [2*epn,2]
+  uint16_t* shards;
+  float* wslots;
+  int64_t shard_stride_rows, wslot_stride;
+  int rank, S, H, K, R, NvS, groups, tok_blocks, zblocks_per_group;
+  unsigned flags;
+};
+
+// NV > 0: the row is exactly NV 16-byte vectors per lane and lives in
+// registers; NV == 0: any H % 8 == 0, strided loop.
+template <int NV>
+__global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int H = a.H;
+  const size_t row_bytes = (size_t)H * 2;
+  if ((int)blockIdx.x < a.tok_blocks) {
+    const int s = blockIdx.x * kWavesPerBlock + wave;
+    if (s >= a.S) return;
+    const int K = a.K;
+    // lane k owns entry (s,k): decode, scatter its weight, publish its row address
+    int dv = 0;
+    if (lane < K) dv = a.dst[(size_t)s * K + lane];
+    const int raw = dv < 0 ? -dv - 1 : dv;
+    const int drank = raw / a.NvS;
+    const int loff = raw - drank * a.NvS;
+    const bool valid = lane < K && drank < a.R;  // never write outside the shards
+    const bool copy = valid && (dv >= 0 || (a.flags & MEP_DISPATCH_WRITE_DUPS));
+    if (valid && a.w) a.wslots[(size_t)drank * a.wslot_stride + loff] = a.w[(size_t)s * K + lane];
+    const uint64_t off = ((uint64_t)drank * (uint64_t)a.shard_stride_rows + (uint64_t)loff) * row_bytes;
+    const uint32_t off_lo = (uint32_t)off, off_hi = (uint32_t)(off >> 32);
+    uint64_t todo = __ballot(copy);
+    const char* src = (const char*)a.hidden + (size_t)s * row_bytes;
+    char* out = (char*)a.shards;
+    if (NV > 0) {
+      mep_u4 v[NV > 0 ? NV : 1];
+#pragma unroll
+      for (int i = 0; i < NV; ++i) v[i] = mep_ld16_stream(src + ((size_t)i * 64 + lane) * 16);
+      while (todo) {
+        const int k = __ffsll((unsigned long long)todo) - 1;
+        todo &= todo - 1;
+        const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(off_hi, k) << 32) |
+                           (uint32_t)__builtin_amdgcn_readlane(off_lo, k);
+        char* row = out + o;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) mep_st16_stream(row + ((size_t)i * 64 + lane) * 16, v[i]);
+      }
+    } else {
+      const int nvec = H / 8;
+      for (int c0 = 0; c0 < nvec; c0 += 4 * 64) {
+        mep_u4 v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c = c0 + i * 64 + lane;
+          if (c < nvec) v[i] = mep_ld16_stream(src + (size_t)c * 16);
+        }
+        uint64_t t = todo;
+        while (t) {
+          const int k = __ffsll((unsigned long long)t) - 1;
+          t &= t - 1;
+          const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(off_hi, k) << 32) |
+                             (uint32_t)__builtin_amdgcn_readlane(off_lo, k);
+          char* row = out + o;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int c = c0 + i * 64 + lane;
+            if (c < nvec) mep_st16_stream(row + (size_t)c * 16, v[i]);
+          }
+        }
+      }
+    }
+    return;
+  }
+  // ---- zero-fill of this rank's padding rows (and their weight slots) -----
+  const int zb = blockIdx.x - a.tok_blocks;
+  const int g = zb / a.zblocks_per_group;
+  const int part = zb - g * a.zblocks_per_group;
+  if (g >= a.groups) return;
+  const int pad_start = a.zero_fill[2 * g];
+  int n_pad = a.zero_fill[2 * g + 1];
+  if (n_pad <= 0 || pad_start < 0) return;
+  if ((int64_t)pad_start + n_pad > a.NvS) n_pad = a.NvS - pad_start;
+  const mep_u4 zero = {0u, 0u, 0u, 0u};
+  const int nvec = H / 8;
+  for (int j = part * kWavesPerBlock + wave; j < n_pad; j += a.zblocks_per_group * kWavesPerBlock) {
+    const int loff = pad_start + j;
+    char* row = (char*)a.shards +
+                ((uint64_t)a.rank * (uint64_t)a.shard_stride_rows + (uint64_t)loff) * row_bytes;
+    for (int c = lane; c < nvec; c += 64) mep_st16_stream(row + (size_t)c * 16, zero);
+    if (a.w && lane == 0) a.wslots[(size_t)a.rank * a.wslot_stride + loff] = 0.0f;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// duplicate groups of one destination rank from every source rank's dst
+// ---------------------------------------------------------------------------
+// pass 1: per (source rank, token): how many of its K entries land on `rank`
+// pass 2: exclusive scan of (#groups, #duplicates) over the R*S tokens
+// pass 3: emit groups in token order
+struct DedupArgs {
+  const int* dst;  // [R, S*K]
+  int* dup_groups; int* dup_loffs; int* dup_counts;
+  int* tok_dups;   // [R*S]   duplicates of each token on `rank` (entries - 1, >= 0)
+  int* blk_sums;   // [2*nblk] per-block (#groups, #dups), then their exclusive scan
+  int rank, S, K, R, NvS, ntok, nblk;
+};
+
+constexpr int kDedupBlock = 256;
+
+__global__ __launch_bounds__(kDedupBlock) void dedup_count_kernel(DedupArgs a) {
+  __shared__ int s_g[kDedupBlock / 64], s_d[kDedupBlock / 64];
+  const int t = blockIdx.x * kDedupBlock + threadIdx.x;
+  int nd = 0;
+  if (t < a.ntok) {
+    const int* d = a.dst + (size_t)t * a.K;
+    int c = 0;
+    for (int k = 0; k < a.K; ++k) {
+      const int v = d[k];
+      const int raw = v < 0 ? -v - 1 : v;
+      c += (raw / a.NvS == a.rank);
+    }
+    nd = c > 1 ? c - 1 : 0;
+    a.tok_dups[t] = nd;
+  }
+  // block totals
+  int g = nd > 0 ? 1 : 0;
+  int gs = mep_wave_incl_scan(g), ds = mep_wave_incl_scan(nd);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 63) { s_g[wave] = gs; s_d[wave] = ds; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int tg = 0, td = 0;
+    for (int w = 0; w < kDedupBlock / 64; ++w) { tg += s_g[w]; td += s_d[w]; }
+    a.blk_sums[2 * blockIdx.x] = tg;
+    a.blk_sums[2 * blockIdx.x + 1] = td;
+  }
+}
+
+// single workgroup: exclusive scan of the per-block sums, totals to dup_counts
+__global__ __launch_bounds__(1024) void dedup_scan_kernel(DedupArgs a) {
+  __shared__ int s_wg[16], s_wd[16];
+  __shared__ int s_carry[2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) { s_carry[0] = 0; s_carry[1] = 0; }
+  __syncthreads();
+  for (int b0 = 0; b0 < a.nblk; b0 += 1024) {
+    const int b = b0 + threadIdx.x;
+    int g = 0, d = 0;
+    if (b < a.nblk) { g = a.blk_sums[2 * b]; d = a.blk_sums[2 * b + 1]; }
+    const int gi = mep_wave_incl_scan(g), di = mep_wave_incl_scan(d);
+    if (lane == 63) { s_wg[wave] = gi; s_wd[wave] = di; }
+    __syncthreads();
+    int og = s_carry[0], od = s_carry[1];
+    for (int w = 0; w < wave; ++w) { og += s_wg[w]; od += s_wd[w]; }
+    if (b < a.nblk) { a.blk_sums[2 * b] = og + gi - g; a.blk_sums[2 * b + 1] = od + di - d; }
+    __syncthreads();
+    if (threadIdx.x == 1023) { s_carry[0] = og + gi; s_carry[1] = od + di; }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) { a.dup_counts[0] = s_carry[0]; a.dup_counts[1] = s_carry[1]; }
+}
+
+__global__ __launch_bounds__(kDedupBlock) void dedup_emit_kernel(DedupArgs a) {
+  __shared__ int s_g[kDedupBlock / 64], s_d[kDedupBlock / 64];
+  const int t = blockIdx.x * kDedupBlock + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nd = t < a.ntok ? a.tok_dups[t] : 0;
+  const int g = nd > 0 ? 1 : 0;
+  const int gi = mep_wave_incl_scan(g), di = mep_wave_incl_scan(nd);
+  if (lane == 63) { s_g[wave] = gi; s_d[wave] = di; }
+  __syncthreads();
+  int og = a.blk_sums[2 * blockIdx.x], od = a.blk_sums[2 * blockIdx.x + 1];
+  for (int w = 0; w < wave; ++w) { og += s_g[w]; od += s_d[w]; }
+  if (nd > 0) {
+    const int gidx = og + gi - 1;
+    int dpos = od + di - nd;
+    const int* d = a.dst + (size_t)t * a.K;
+    bool first = true;
+    for (int k = 0; k < a.K; ++k) {
+      const int v = d[k];
+      const int raw = v < 0 ? -v - 1 : v;
+      const int dr = raw / a.NvS;
+      if (dr != a.rank) continue;
+      const int loff = raw - dr * a.NvS;
+      if (first) {
+        a.dup_groups[3 * gidx] = loff;
+        a.dup_groups[3 * gidx + 1] = dpos;
+        a.dup_groups[3 * gidx + 2] = nd;
+        first = false;
+      } else {
+        a.dup_loffs[dpos++] = loff;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// duplicate expansion / pre-reduction on one shard: one wave per group
+// ---------------------------------------------------------------------------
+struct DupArgs {
+  uint16_t* shard;
+  const int* dup_groups; const int* dup_loffs; const int* dup_counts;
+  int NvS, H;
+};
+
+__global__ __launch_bounds__(kBlock) void epilogue_kernel(DupArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int nw = gridDim.x * kWavesPerBlock;
+  int ng = a.dup_counts[0];
+  if (ng > a.NvS) ng = a.NvS;
+  const size_t row_bytes = (size_t)a.H * 2;
+  const int nvec = a.H / 8;
+  for (int g = gw; g < ng; g += nw) {
+    const int p = a.dup_groups[3 * g], start = a.dup_groups[3 * g + 1], n = a.dup_groups[3 * g + 2];
+    if ((unsigned)p >= (unsigned)a.NvS || start < 0 || n <= 0 || (int64_t)start + n > a.NvS) continue;
+    const char* src = (const char*)a.shard + (size_t)p * row_bytes;
+    for (int c0 = 0; c0 < nvec; c0 += 4 * 64) {
+      mep_u4 v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = c0 + i * 64 + lane;
+        if (c < nvec) v[i] = mep_ld16(src + (size_t)c * 16);
+      }
+      for (int j = 0; j < n; ++j) {
+        const int lo = a.dup_loffs[start + j];
+        if ((unsigned)lo >= (unsigned)a.NvS) continue;
+        char* row = (char*)a.shard + (size_t)lo * row_bytes;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c = c0 + i * 64 + lane;
+          if (c < nvec) mep_st16(row + (size_t)c * 16, v[i]);
+        }
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void prologue_kernel(DupArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int nw = gridDim.x * kWavesPerBlock;
+  int ng = a.dup_counts[0];
+  if (ng > a.NvS) ng = a.NvS;
+  const size_t row_bytes = (size_t)a.H * 2;
+  const int nvec = a.H / 8;
+  for (int g = gw; g < ng; g += nw) {
+    const int p = a.dup_groups[3 * g], start = a.dup_groups[3 * g + 1], n = a.dup_groups[3 * g + 2];
+    if ((unsigned)p >= (unsigned)a.NvS || start < 0 || n <= 0 || (int64_t)start + n > a.NvS) continue;
+    char* prow = (char*)a.shard + (size_t)p * row_bytes;
+    for (int c = lane; c < nvec; c += 64) {
+      float acc[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+      mep_u4 v = mep_ld16(prow + (size_t)c * 16);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { acc[2 * i] += mep_bf16_lo(v[i]); acc[2 * i + 1] += mep_bf16_hi(v[i]); }
+      for (int j = 0; j < n; ++j) {
+        const int lo = a.dup_loffs[start + j];
+        if ((unsigned)lo >= (unsigned)a.NvS) continue;
+        v = mep_ld16((const char*)a.shard + (size_t)lo * row_bytes + (size_t)c * 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { acc[2 * i] += mep_bf16_lo(v[i]); acc[2 * i + 1] += mep_bf16_hi(v[i]); }
+      }
+      mep_u4 o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = mep_pack_bf16(acc[2 * i], acc[2 * i + 1]);
+      mep_st16(prow + (size_t)c * 16, o);
+    }
+  }
+}
+
+int dup_grid(int NvS) {
+  int blocks = (NvS + kWavesPerBlock - 1) / kWavesPerBlock;
+  return blocks < 2048 ? (blocks > 0 ? blocks : 1) : 2048;
+}
+
+}  // namespace
+
+extern "C" int mep_dispatch(const void* hidden_SH, const float* w_SK, const int32_t* dst,
+                            const int32_t* zero_fill, void* shards, int64_t shard_stride_rows,
+                            float* wslots, int64_t wslot_stride, int rank, int S, int H, int K,
+                            int R, int epn, int NvS, int token_padding, unsigned flags,
+                            void* stream) {
+  MEP_REQUIRE(hidden_SH && dst && shards, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE((w_SK == nullptr) == (wslots == nullptr), MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(S > 0 && H > 0 && K > 0 && R > 0 && epn > 0 && NvS > 0 && token_padding > 0,
+              MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(rank >= 0 && rank < R, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(K <= 32, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(H % 8 == 0, MEP_ERR_UNSUPPORTED);  // 16-byte row vectors (reference dispatch.py:901)
+  MEP_REQUIRE(shard_stride_rows >= NvS && (!wslots || wslot_stride >= NvS), MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(((uintptr_t)hidden_SH % 16 == 0) && ((uintptr_t)shards % 16 == 0), MEP_ERR_ALIGNMENT);
+  const bool zf = zero_fill && !(flags & MEP_DISPATCH_NO_ZERO_FILL);
+  DispatchArgs a;
+  a.hidden = (const uint16_t*)hidden_SH; a.w = w_SK; a.dst = dst; a.zero_fill = zero_fill;
+  a.shards = (uint16_t*)shards; a.wslots = wslots;
+  a.shard_stride_rows = shard_stride_rows; a.wslot_stride = wslot_stride;
+  a.rank = rank; a.S = S; a.H = H; a.K = K; a.R = R; a.NvS = NvS; a.flags = flags;
+  a.groups = zf ? 2 * epn : 0;
+  a.tok_blocks = (S + kWavesPerBlock - 1) / kWavesPerBlock;
+  int zpg = (token_padding - 1 + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (zpg > 32) zpg = 32;
+  if (zpg < 1) zpg = 1;
+  a.zblocks_per_group = zpg;
+  const int zblocks = (zf && token_padding > 1) ? a.groups * zpg : 0;
+  if (zblocks == 0) a.groups = 0;
+  dim3 grid(a.tok_blocks + zblocks);
+  hipStream_t st = (hipStream_t)stream;
+  const int nvec = H / 8;
+  if (nvec % 64 == 0 && nvec / 64 == 14) {
+    hipLaunchKernelGGL(dispatch_kernel<14>, grid, dim3(kBlock), 0, st, a);
+  } else if (nvec % 64 == 0 && nvec / 64 == 8) {
+    hipLaunchKernelGGL(dispatch_kernel<8>, grid, dim3(kBlock), 0, st, a);
+  } else {
+    hipLaunchKernelGGL(dispatch_kernel<0>, grid, dim3(kBlock), 0, st, a);
+  }
+  return mep_launch_status();
+}
+
+extern "C" size_t mep_dedup_scratch_bytes(int S, int R) {
+  if (S <= 0 || R <= 0) return 0;
+  const size_t ntok = (size_t)S * R;
+  const size_t nblk = (ntok + kDedupBlock - 1) / kDedupBlock;
+  return (ntok + 2 * nblk) * sizeof(int);
+}
+
+extern "C" int mep_build_dedup(const int32_t* dst_RN, int rank, int S, int K, int R, int NvS,
+                               int32_t* dup_groups, int32_t* dup_loffs, int32_t* dup_counts,
+                               void* scratch, size_t scratch_bytes, void* stream) {
+  MEP_REQUIRE(dst_RN && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(S > 0 && K > 0 && R > 0 && NvS > 0 && rank >= 0 && rank < R, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE((int64_t)S * R < INT32_MAX, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(scratch && scratch_bytes >= mep_dedup_scratch_bytes(S, R), MEP_ERR_SCRATCH);
+  DedupArgs a;
+  a.dst = dst_RN; a.dup_groups = dup_groups; a.dup_loffs = dup_loffs; a.dup_counts = dup_counts;
+  a.rank = rank; a.S = S; a.K = K; a.R = R; a.NvS = NvS;
+  a.ntok = S * R;
+  a.nblk = (a.ntok + kDedupBlock - 1) / kDedupBlock;
+  a.tok_dups = (int*)scratch;
+  a.blk_sums = a.tok_dups + a.ntok;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(dedup_count_kernel, dim3(a.nblk), dim3(kDedupBlock), 0, st, a);
+  hipLaunchKernelGGL(dedup_scan_kernel, dim3(1), dim3(1024), 0, st, a);
+  hipLaunchKernelGGL(dedup_emit_kernel, dim3(a.nblk), dim3(kDedupBlock), 0, st, a);
+  return mep_launch_status();
+}
+
+extern "C" int mep_dispatch_epilogue(void* shard, const int32_t* dup_groups,
+                                     const int32_t* dup_loffs, const int32_t* dup_counts, int NvS,
+                                     int H, void* stream) {
+  MEP_REQUIRE(shard && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(NvS > 0 && H > 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(H % 8 == 0, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((uintptr_t)shard % 16 == 0, MEP_ERR_ALIGNMENT);
+  DupArgs a{(uint16_t*)shard, dup_groups, dup_loffs, dup_counts, NvS, H};
+  hipLaunchKernelGGL(epilogue_kernel, dim3(dup_grid(NvS)), dim3(kBlock), 0, (hipStream_t)stream, a);
+  return mep_launch_status();
+}
+
+extern "C" int mep_combine_prologue(void* shard, const int32_t* dup_groups,
+                                    const int32_t* dup_loffs, const int32_t* dup_counts, int NvS,
+                                    int H, void* stream) {
+  MEP_REQUIRE(shard && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(NvS > 0 && H > 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(H % 8 == 0, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((uintptr_t)shard % 16 == 0, MEP_ERR_ALIGNMENT);
+  DupArgs a{(uint16_t*)shard, dup_groups, dup_loffs, dup_counts, NvS, H};
+  hipLaunchKernelGGL(prologue_kernel, dim3(dup_grid(NvS)), dim3(kBlock), 0, (hipStream_t)stream, a);
+  return mep_launch_status();
+}

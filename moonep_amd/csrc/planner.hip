@@ -1,0 +1,359 @@
+// Online redundant-expert planner for gfx950.
+//
+// One kernel, no grid-wide synchronisation: every workgroup rebuilds the
+// (tiny, rank-independent) balancing plan in its own LDS from the R x E count
+// matrix and then resolves the slots of its own slice of the rank's S*K
+// routed entries.  Rebuilding the plan per workgroup costs nothing in latency
+// (workgroups run side by side on different CUs) and removes the reference's
+// rank-0 stage, its broadcast and its three barriers
+// (reference moonep/planning.py:577-583, 917-922, 941, 1045).
+//
+// Results are bit-identical to the reference oracle
+// (reference tests/planning_reference.py:25-311).
+#include "mep_common.h"
+
+namespace {
+
+struct PlanArgs {
+  const int* tpe;    // [R,E]
+  const int* topk;   // [nranks, S*K]
+  int* dst;          // [nranks, S*K]
+  int* cu_seqlens;   // [nranks, 2*epn]
+  int* etc;          // [R, epn]
+  int* zero_fill;    // [nranks, 2*epn, 2]
+  int* remote_stats; // [nranks, 2]
+  int* scratch;      // alloc/base tables when they do not fit in LDS
+  int rank0, S, K, E, R, epn, tp, NvS, tok_per_wg;
+};
+
+// LDS layout in ints (must match plan_lds_ints on the host)
+template <int NT>
+struct PlanLds {
+  static constexpr int NW = NT / MEP_WAVE;
+  static constexpr int W4 = (NW + 3) / 4;  // packed per-wave byte counters per expert
+  static constexpr int E_ARRAYS = 5 + W4;
+  static constexpr int R_ARRAYS = 6;
+  static constexpr int FIXED = 2 * NT;
+};
+
+template <int NT, bool kLdsTables>
+__global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
+  using L = PlanLds<NT>;
+  constexpr int NW = L::NW;
+  constexpr int W4 = L::W4;
+  extern __shared__ int smem[];
+  const int E = a.E, R = a.R, epn = a.epn, tp = a.tp, NvS = a.NvS, K = a.K;
+  const int N = a.S * K;
+  const int CAP = N;
+  int* s_cnt = smem;             // [E] tokens per expert, all ranks
+  int* s_prev = s_cnt + E;       // [E] tokens of the ranks before this one
+  int* s_rem = s_prev + E;       // [E] not yet migrated
+  int* s_etc = s_rem + E;        // [R*epn] remote experts per destination
+  int* s_hist = s_etc + E;       // [E] entries of this rank before my slice
+  int* s_wcnt = s_hist + E;      // [E*W4] per-wave counts, one byte per wave
+  int* s_gt = s_wcnt + W4 * E;   // [R] tokens per home group
+  int* s_from = s_gt + R;        // [R] donor feeding this receiver (-1: none)
+  int* s_quota = s_from + R;     // [R] tokens still to receive
+  int* s_stat1 = s_quota + R;    // [R] slots elsewhere holding my experts
+  int* s_nrem = s_stat1 + R;     // [R] remote experts on this destination
+  int* s_bal = s_nrem + R;       // [R]
+  int* s_ce = s_bal + R;         // [NT] expert of each entry of my slice
+  int* s_cd = s_ce + NT;         // [NT] destination rank of each entry
+  int* tbl = kLdsTables ? (s_cd + NT)
+                        : a.scratch + (size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 2 * E * R;
+  int* alloc = tbl;            // [E,R] tokens of e on d, later its prefix over d
+  int* base = tbl + E * R;     // [E,R] dst = base[e,d] + global index of the entry
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int rank = a.rank0 + blockIdx.y;
+  const bool writer = blockIdx.x == 0;  // one workgroup per rank stores the small outputs
+
+  // ---- counts per expert, per home group --------------------------------
+  for (int i = tid; i < R; i += NT) {
+    s_gt[i] = 0; s_from[i] = -1; s_quota[i] = 0; s_stat1[i] = 0; s_nrem[i] = 0;
+  }
+  for (int i = tid; i < W4 * E; i += NT) s_wcnt[i] = 0;
+  for (int i = tid; i < E; i += NT) s_hist[i] = 0;
+  __syncthreads();
+  for (int e = tid; e < E; e += NT) {
+    int c = 0, p = 0;
+    for (int r = 0; r < R; ++r) {
+      int v = a.tpe[r * E + e];
+      if (r < rank) p += v;
+      c += v;
+    }
+    s_cnt[e] = c; s_prev[e] = p; s_rem[e] = c;
+    const int home = e / epn;
+    for (int d = 0; d < R; ++d) alloc[e * R + d] = (d == home) ? c : 0;
+    atomicAdd(&s_gt[home], c);
+  }
+  __syncthreads();
+
+  // ---- receivers and quotas: one wave, balances in registers -------------
+  // Each receiver is filled exactly once (to capacity), so z[h][u] of the
+  // reference (tests/planning_reference.py:85-96) is stored per receiver.
+  if (wave == 0) {
+    int b0 = lane < R ? s_gt[lane] - CAP : 0;
+    int b1 = lane + 64 < R ? s_gt[lane + 64] - CAP : 0;
+    const bool v0 = lane < R, v1 = lane + 64 < R;
+    for (int it = 0; it < R; ++it) {
+      // candidate of this lane for max (first index wins ties) and min
+      int mx = v0 ? b0 : INT32_MIN, mxi = lane;
+      if (v1 && b1 > mx) { mx = b1; mxi = lane + 64; }
+      int mn = v0 ? b0 : INT32_MAX, mni = lane;
+      if (v1 && b1 < mn) { mn = b1; mni = lane + 64; }
+      int hv, h, uv, u;
+      mep_wave_argmax_first(mx, mxi, hv, h);
+      mep_wave_argmin_first(mn, mni, uv, u);
+      if (hv <= 0 || uv >= 0) break;
+      const int move = -uv;
+      if (lane == (h & 63)) { if (h < 64) b0 -= move; else b1 -= move; }
+      if (lane == (u & 63)) { if (u < 64) b0 = 0; else b1 = 0; }
+      if (lane == 0) { s_from[u] = h; s_quota[u] = move; }
+    }
+  }
+  __syncthreads();
+
+  // ---- which tokens of which expert migrate: one wave per home group -----
+  for (int h = wave; h < R; h += NW) {
+    const int es = h * epn;
+    for (int it = 0; it < R + epn; ++it) {
+      int q = INT32_MIN, qi = INT32_MAX;
+      for (int d = lane; d < R; d += 64) {
+        int v = (s_from[d] == h) ? s_quota[d] : 0;
+        if (v > q) { q = v; qi = d; }
+      }
+      int quota, d;
+      mep_wave_argmax_first(q, qi, quota, d);
+      if (quota <= 0) break;
+      int rm = INT32_MIN, ri = INT32_MAX;
+      for (int le = lane; le < epn; le += 64) {
+        int v = s_rem[es + le];
+        if (v > rm) { rm = v; ri = le; }
+      }
+      int rem, le;
+      mep_wave_argmax_first(rm, ri, rem, le);
+      if (rem <= 0) break;
+      const int take = rem < quota ? rem : quota;
+      if (lane == 0) {
+        const int e = es + le;
+        alloc[e * R + d] += take;
+        alloc[e * R + h] -= take;
+        s_rem[e] = rem - take;
+        s_quota[d] = quota - take;
+      }
+      mep_wave_sync();
+    }
+  }
+  __syncthreads();
+
+  // ---- layout of every destination: one wave per destination -------------
+  for (int d = wave; d < R; d += NW) {
+    const int lo = d * epn, hi = lo + epn;
+    int nremote = 0;
+    for (int c = 0; c < E; c += 64) {
+      const int e = c + lane;
+      const bool sel = e < E && (e < lo || e >= hi) && alloc[e * R + d] > 0;
+      const uint64_t m = __ballot(sel);
+      if (sel) {
+        const int slot = nremote + __popcll(m & mep_lanes_lt());
+        if (slot < epn) s_etc[lo + slot] = e;
+        atomicAdd(&s_stat1[e / epn], 1);
+      }
+      nremote += __popcll(m);
+    }
+    for (int b = nremote + lane; b < epn; b += 64) s_etc[lo + b] = -1;
+    if (lane == 0) s_nrem[d] = nremote;
+    mep_wave_sync();
+    const bool mine = writer && d == rank;
+    int* cu = a.cu_seqlens + (size_t)blockIdx.y * 2 * epn;
+    int* zf = a.zero_fill + (size_t)blockIdx.y * 4 * epn;
+    int running = 0;
+    for (int c = 0; c < 2 * epn; c += 64) {
+      const int g = c + lane;
+      int eid = -1, cnt = 0;
+      if (g < epn) eid = lo + g;
+      else if (g < 2 * epn) eid = s_etc[lo + g - epn];
+      if (eid >= 0) cnt = alloc[eid * R + d];
+      const int padded = cnt > 0 ? ((cnt + tp - 1) / tp) * tp : 0;
+      const int incl = mep_wave_incl_scan(padded);
+      const int start = running + incl - padded;
+      if (cnt > 0) base[eid * R + d] = d * NvS + start;
+      if (mine && g < 2 * epn) {
+        cu[g] = start + padded;
+        zf[2 * g] = padded > cnt ? start + cnt : 0;
+        zf[2 * g + 1] = padded - cnt;
+      }
+      running += __builtin_amdgcn_readlane(incl, 63);
+    }
+  }
+  __syncthreads();
+
+  if (writer) {
+    if (blockIdx.y == 0)
+      for (int i = tid; i < R * epn; i += NT) a.etc[i] = s_etc[i];
+    if (tid == 0) {
+      a.remote_stats[2 * blockIdx.y] = s_nrem[rank];
+      a.remote_stats[2 * blockIdx.y + 1] = s_stat1[rank];
+    }
+  }
+
+  // ---- prefix over destinations; fold it into the slot base --------------
+  for (int e = tid; e < E; e += NT) {
+    int run = 0;
+    for (int d = 0; d < R; ++d) {
+      const int v = alloc[e * R + d];
+      base[e * R + d] -= run;
+      run += v;
+      alloc[e * R + d] = run;
+    }
+  }
+
+  // ---- my slice of the rank's entries -------------------------------------
+  const int* topk = a.topk + (size_t)blockIdx.y * N;
+  int* dst = a.dst + (size_t)blockIdx.y * N;
+  const int t0 = blockIdx.x * a.tok_per_wg;
+  const int t1 = min(t0 + a.tok_per_wg, a.S);
+  const int e0 = t0 * K;
+  const int n = (t1 - t0) * K;  // <= NT
+
+  // entries before my slice, per expert
+  for (int i = tid; i < e0; i += NT) {
+    const int e = topk[i];
+    if ((unsigned)e < (unsigned)E) atomicAdd(&s_hist[e], 1);
+  }
+  int e = -1;
+  if (tid < n) {
+    e = topk[e0 + tid];
+    if ((unsigned)e >= (unsigned)E) e = -1;  // invalid id: slot 0, never out of bounds
+  }
+  // position among equal experts inside my wave
+  int pos = 0;
+  {
+    uint64_t todo = __ballot(e >= 0);
+    while (todo) {
+      const int leader = __ffsll((unsigned long long)todo) - 1;
+      const int ev = __builtin_amdgcn_readlane(e, leader);
+      const uint64_t m = __ballot(e == ev);
+      if (e == ev) {
+        pos = __popcll(m & mep_lanes_lt());
+        if (pos == 0) atomicAdd(&s_wcnt[e * W4 + (wave >> 2)], __popcll(m) << (8 * (wave & 3)));
+      }
+      todo &= ~m;
+    }
+  }
+  __syncthreads();
+  int dv = 0, dest = 0;
+  if (e >= 0) {
+    int before = 0;
+    for (int w4 = 0; w4 <= (wave >> 2); ++w4) {
+      const unsigned word = (unsigned)s_wcnt[e * W4 + w4];
+      for (int b = 0; b < 4; ++b)
+        if (w4 * 4 + b < wave) before += (word >> (8 * b)) & 0xffu;
+    }
+    const int g = s_prev[e] + s_hist[e] + before + pos;
+    while (dest < R - 1 && alloc[e * R + dest] <= g) ++dest;
+    dv = base[e * R + dest] + g;
+  }
+  s_cd[tid] = dest;
+  __syncthreads();
+  if (tid < n) {
+    const int k = tid % K;
+    bool dup = false;
+    for (int j = tid - k; j < tid; ++j) dup |= (s_cd[j] == dest);
+    dst[e0 + tid] = dup ? -dv - 1 : dv;
+  }
+}
+
+size_t plan_lds_bytes(int nt, int E, int R, bool lds_tables) {
+  const int nw = nt / MEP_WAVE;
+  const int w4 = (nw + 3) / 4;
+  size_t ints = (size_t)(5 + w4) * E + 6 * (size_t)R + 2 * (size_t)nt;
+  if (lds_tables) ints += 2 * (size_t)E * R;
+  return ints * sizeof(int);
+}
+
+constexpr size_t kLdsDefaultLimit = 64 * 1024;
+
+struct PlanConfig {
+  int nt;
+  bool lds_tables;
+  size_t lds_bytes;
+  int tok_per_wg;
+  int groups;
+};
+
+// 0 on success
+int plan_config(int S, int K, int E, int R, PlanConfig* c) {
+  if (plan_lds_bytes(1024, E, R, true) <= kLdsDefaultLimit) {
+    c->nt = 1024; c->lds_tables = true;
+  } else if (plan_lds_bytes(256, E, R, true) <= kLdsDefaultLimit) {
+    c->nt = 256; c->lds_tables = true;
+  } else if (plan_lds_bytes(256, E, R, false) <= kLdsDefaultLimit) {
+    c->nt = 256; c->lds_tables = false;
+  } else {
+    return MEP_ERR_UNSUPPORTED;
+  }
+  c->lds_bytes = plan_lds_bytes(c->nt, E, R, c->lds_tables);
+  c->tok_per_wg = c->nt / K;
+  c->groups = (S + c->tok_per_wg - 1) / c->tok_per_wg;
+  return MEP_OK;
+}
+
+}  // namespace
+
+extern "C" size_t mep_plan_scratch_bytes(int S, int K, int E, int R, int nranks) {
+  PlanConfig c;
+  if (S <= 0 || K <= 0 || K > 32 || E <= 0 || R <= 0 || nranks <= 0) return 0;
+  if (plan_config(S, K, E, R, &c) != MEP_OK || c.lds_tables) return 0;
+  return (size_t)c.groups * nranks * 2 * (size_t)E * R * sizeof(int);
+}
+
+extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int nranks,
+                              int S, int K, int E, int R, int token_padding, int NvS, int32_t* dst,
+                              int32_t* cu_seqlens, int32_t* experts_to_copy, int32_t* zero_fill,
+                              int32_t* remote_stats, void* scratch, size_t scratch_bytes,
+                              void* stream) {
+  MEP_REQUIRE(tpe_RE && topk_nSK && dst && cu_seqlens && experts_to_copy && zero_fill &&
+                  remote_stats, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(S > 0 && K > 0 && E > 0 && R > 0 && token_padding > 0 && NvS > 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(E % R == 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(nranks > 0 && rank0 >= 0 && rank0 + nranks <= R, MEP_ERR_INVALID_ARG);
+  // encoding bounds of the reference (moonep/planning.py:1231-1255, api.py:286-290)
+  MEP_REQUIRE(K <= 32 && R <= 128, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((int64_t)S * K < INT32_MAX && (int64_t)S * K <= NvS, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((int64_t)R * NvS <= INT32_MAX, MEP_ERR_UNSUPPORTED);
+  PlanConfig c;
+  int rc = plan_config(S, K, E, R, &c);
+  if (rc != MEP_OK) return rc;
+  if (!c.lds_tables) {
+    const size_t need = (size_t)c.groups * nranks * 2 * (size_t)E * R * sizeof(int);
+    MEP_REQUIRE(scratch && scratch_bytes >= need, MEP_ERR_SCRATCH);
+  }
+  PlanArgs a;
+  a.tpe = tpe_RE; a.topk = topk_nSK; a.dst = dst; a.cu_seqlens = cu_seqlens;
+  a.etc = experts_to_copy; a.zero_fill = zero_fill; a.remote_stats = remote_stats;
+  a.scratch = (int*)scratch;
+  a.rank0 = rank0; a.S = S; a.K = K; a.E = E; a.R = R; a.epn = E / R; a.tp = token_padding;
+  a.NvS = NvS; a.tok_per_wg = c.tok_per_wg;
+  dim3 grid(c.groups, nranks);
+  hipStream_t st = (hipStream_t)stream;
+  if (c.nt == 1024) {
+    hipLaunchKernelGGL((plan_kernel<1024, true>), grid, dim3(1024), c.lds_bytes, st, a);
+  } else if (c.lds_tables) {
+    hipLaunchKernelGGL((plan_kernel<256, true>), grid, dim3(256), c.lds_bytes, st, a);
+  } else {
+    hipLaunchKernelGGL((plan_kernel<256, false>), grid, dim3(256), c.lds_bytes, st, a);
+  }
+  return mep_launch_status();
+}
+
+extern "C" int mep_plan(const int32_t* tpe_RE, const int32_t* topk_SK, int rank, int S, int K,
+                        int E, int R, int token_padding, int NvS, int32_t* dst,
+                        int32_t* cu_seqlens, int32_t* experts_to_copy, int32_t* zero_fill,
+                        int32_t* remote_stats, void* scratch, size_t scratch_bytes, void* stream) {
+  return mep_plan_ranks(tpe_RE, topk_SK, rank, 1, S, K, E, R, token_padding, NvS, dst, cu_seqlens,
+                        experts_to_copy, zero_fill, remote_stats, scratch, scratch_bytes, stream);
+}
