@@ -1,0 +1,300 @@
+"""Headline benchmark: one rank's share of plan -> dispatch -> combine on one
+MI355X at S=4096, H=7168, K=8, E=256, R=8, token_padding=128, bf16, routing at
+maxvio ~= 1 (synthetic, seeded).
+
+    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--full]
+
+A step is one replay of a HIP graph holding the three launches (planner,
+dispatch, combine).  Prints ONE JSON line.  `value` is the chain's throughput:
+algorithmic bytes of dispatch + combine (each S*H*2 + S*K*H*2) divided by the
+time of a whole step (planner included), in GB/s, inputs resident in HBM.
+Per-kernel durations are measured with HIP events on the launching stream;
+the dominant kernel's figure feeds `roofline`.  `--full` adds the maxvio
+sweep, the second shape, prefetch_weight and reduce_grad to the JSON line.
+
+The CPU baseline is the scalar C restatement of the same chain
+(oracle/mep_oracle.c), timed on the host next to the GPU.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs scaled by a plain copy kernel; the summary that holds them is
+# profiles/dispatch_combine_main_pmc.md.  None until measured.
+MEASURED_TRAFFIC_BYTES = {"dispatch": None, "combine": None}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--full", action="store_true", help="also sweep maxvio, 2nd shape, prefetch, grad reduce")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--maxvio", type=float, default=1.0)
+    ap.add_argument("--seed", type=int, default=2024)
+    return ap.parse_args()
+
+
+def time_launches(fn, iters, warmup=2):
+    """Average duration in microseconds of `fn`'s work on the current stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) * 1e3 / iters
+
+
+class Chain:
+    """plan -> dispatch -> combine of one rank on its real shapes."""
+
+    def __init__(self, S, H, K, E, R, tp, rank, maxvio, seed, nsets=2):
+        import torch
+
+        from moonep_amd import Buffer, routing
+        from moonep_amd.combine import launch_combine
+        from moonep_amd.dispatch import launch_dispatch
+        from moonep_amd.planning import allocate_planning_outputs, launch_planning
+
+        self.S, self.H, self.K, self.E, self.R = S, H, K, E, R
+        dev = torch.device("cuda", 0)
+        topk, w, tpe, self.maxvio, self.sigma = routing.logit_routing(S, K, E, R, maxvio, seed)
+        self.topk_all, self.tpe_cpu, self.w_cpu = topk, tpe, w
+        self.buf = Buffer(S, H, K, E, R, token_padding=tp, rank=rank)
+        self.ctx = ctx = self.buf._require_ctx()
+        self.rank = rank
+        self.topk = topk[rank].reshape(-1).contiguous().to(dev)
+        self.tpe = tpe.to(dev)
+        self.wk = w[rank].contiguous().to(dev)
+        g = torch.Generator().manual_seed(seed + 99)
+        # several input/output sets so that a replay never finds its tokens in cache
+        self.hidden = [torch.randn(S, H, generator=g).to(torch.bfloat16).to(dev) for _ in range(nsets)]
+        self.out = [torch.empty(S, H, dtype=torch.bfloat16, device=dev) for _ in range(nsets)]
+        self.out_w = torch.empty(S, K, dtype=torch.float32, device=dev)
+        self.plan, self.cu = allocate_planning_outputs(ctx)
+        ctx["hidden_buf"].zero_()
+
+        def plan_fn():
+            launch_planning(ctx, self.topk, self.tpe, self.cu, self.plan)
+
+        def dispatch_fn(i=0):
+            launch_dispatch(ctx, self.hidden[i], self.wk, self.plan, build_dedup_map=False,
+                            write_dups=True)
+
+        def combine_fn(i=0):
+            launch_combine(ctx, self.out[i], self.plan.dst, self.out_w, mode="two_level")
+
+        self.plan_fn, self.dispatch_fn, self.combine_fn = plan_fn, dispatch_fn, combine_fn
+        # eager once (also validates), then capture one graph per buffer set
+        plan_fn(); dispatch_fn(); combine_fn()
+        torch.cuda.synchronize()
+        self.graphs = []
+        for i in range(nsets):
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                plan_fn(); dispatch_fn(i); combine_fn(i)
+            self.graphs.append(gr)
+        torch.cuda.synchronize()
+
+    def bytes_one_way(self):
+        return self.S * self.H * 2 + self.S * self.K * self.H * 2
+
+    def step(self, i):
+        self.graphs[i % len(self.graphs)].replay()
+
+    def destroy(self):
+        self.graphs = []
+        self.buf.destroy()
+
+
+def measure_chain(ch, steps, warmup):
+    import torch
+
+    for i in range(warmup):
+        ch.step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(steps):
+        ch.step(i)
+    b.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = a.elapsed_time(b) / steps
+    per = {}
+    n = max(steps, 10)
+    per["plan_us"] = time_launches(ch.plan_fn, n)
+    k = [0]
+
+    def d():
+        k[0] += 1
+        ch.dispatch_fn(k[0] % len(ch.hidden))
+
+    def c():
+        k[0] += 1
+        ch.combine_fn(k[0] % len(ch.out))
+
+    per["dispatch_us"] = time_launches(d, n)
+    per["combine_us"] = time_launches(c, n)
+    by = ch.bytes_one_way()
+    per["dispatch_GBps"] = by / per["dispatch_us"] / 1e3
+    per["combine_GBps"] = by / per["combine_us"] / 1e3
+    return wall_ms, ev_ms, per
+
+
+def cpu_baseline(ch, budget_s=20.0):
+    """Scalar C port of plan + dispatch + combine on the same inputs, host cores."""
+    import numpy as np
+    import torch
+
+    from oracle import c_oracle as co
+
+    S, H, K, E, R = ch.S, ch.H, ch.K, ch.E, ch.R
+    ctx = ch.ctx
+    NvS, tp = int(ctx["NvS"]), int(ctx["token_padding"])
+    topk = ch.topk_all[ch.rank].numpy()
+    tpe = ch.tpe_cpu.numpy()
+    hidden = ch.hidden[0].cpu().view(torch.int16).numpy().view(np.uint16)
+    w = ch.w_cpu[ch.rank].contiguous().numpy()
+    shards = np.empty((R, NvS, H), np.uint16)   # pages are touched only where rows land
+    wslots = np.empty((R, NvS), np.float32)
+    times = []
+    t_all = time.perf_counter()
+    while True:
+        t0 = time.perf_counter()
+        dst, cu, etc, zf, st = co.plan(tpe, topk, ch.rank, S, K, tp, NvS)
+        t1 = time.perf_counter()
+        co.dispatch(hidden, w, dst, zf, shards, wslots, ch.rank, K, NvS, True)
+        t2 = time.perf_counter()
+        out, out_w = co.combine(shards, wslots, dst, S, K, NvS, 2)
+        t3 = time.perf_counter()
+        times.append((t1 - t0, t2 - t1, t3 - t2))
+        if len(times) >= 2 and time.perf_counter() - t_all > budget_s or len(times) >= 8:
+            break
+    # first pass pays the page faults of the fresh shards: report the best later pass
+    p, d, c = min(times[1:], key=lambda t: sum(t))
+    total = p + d + c
+    got = ch.out[0].cpu().view(torch.int16).numpy().view(np.uint16)
+    return {
+        "value": 2 * ch.bytes_one_way() / total / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"full workload (S={S} tokens of one rank), best of {len(times) - 1} passes after 1 warm-up",
+        "plan_us": p * 1e6, "dispatch_GBps": ch.bytes_one_way() / d / 1e9,
+        "combine_GBps": ch.bytes_one_way() / c / 1e9, "host_cpus": os.cpu_count(),
+        "matches_gpu_output": bool(np.array_equal(out, got)),
+    }
+
+
+def bench_weights(seed, steps):
+    """prefetch_weight and reduce_grad, one projection, plan of the main config."""
+    import torch
+
+    from moonep_amd import routing
+    from moonep_amd.grad_reduce import launch_grad_reduce
+    from moonep_amd.prefetch import launch_prefetch
+    from oracle import planner_oracle as po
+
+    S, K, E, R, H, Hp, rank = 4096, 8, 256, 8, 7168, 2048, 0
+    epn = E // R
+    dev = torch.device("cuda", 0)
+    topk, _, tpe, mv, _ = routing.logit_routing(S, K, E, R, 1.0, seed, want_weights=False)
+    gp = po.plan_global(tpe.numpy(), S, K, 128)
+    etc_np = gp.experts_to_copy
+    etc = torch.from_numpy(etc_np.astype("int32")).to(dev)
+    # busiest owner
+    owned = [(int(((etc_np // epn) == r).sum()), r) for r in range(R)]
+    n_slots, rank = max(owned)
+    active = len({int(e) for e in etc_np.reshape(-1) if e >= 0 and e // epn == rank})
+    own_slots = int((etc_np[rank] >= 0).sum())
+    res = {"plan_maxvio": mv, "rank": rank, "slots_pushed": n_slots, "active_experts": active,
+           "own_occupied_slots": own_slots}
+    per = H * Hp
+    local = (torch.randn(epn, H, Hp, device=dev) * 0.02).to(torch.bfloat16)
+    pool = torch.empty(R, epn, H, Hp, dtype=torch.bfloat16, device=dev)
+    us = time_launches(lambda: launch_prefetch((local,) * 3, (pool,) * 3, etc, rank=rank), steps)
+    by = 3 * (active + n_slots) * per * 2
+    res["prefetch_us_3proj"] = us
+    res["prefetch_GBps"] = by / us / 1e3 if n_slots else 0.0
+    res["prefetch_bytes"] = by
+    del local, pool
+    torch.cuda.empty_cache()
+    grad = torch.zeros(epn, H, Hp, dtype=torch.float32, device=dev)
+    red = torch.randn(R, epn, H, Hp, dtype=torch.float32, device=dev) * 1e-3
+    us = time_launches(lambda: launch_grad_reduce(grad, red, etc, rank=rank), steps)
+    by = (n_slots + 2 * active + own_slots) * per * 4
+    res["grad_reduce_us"] = us
+    res["grad_reduce_GBps"] = by / us / 1e3 if by else 0.0
+    res["grad_reduce_bytes"] = by
+    return res
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one rank's share on ONE GPU; --gpus > 1 is not part of this "
+              "build (no collectives, no sharding).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    torch.cuda.set_device(0)
+    S, H, K, E, R, tp, rank = 4096, 7168, 8, 256, 8, 128, 0
+    ch = Chain(S, H, K, E, R, tp, rank, args.maxvio, args.seed)
+    wall_ms, ev_ms, per = measure_chain(ch, args.steps, args.warmup)
+    by = ch.bytes_one_way()
+    value = 2 * by / (wall_ms * 1e-3) / 1e9
+    dom = "dispatch" if per["dispatch_us"] >= per["combine_us"] else "combine"
+    achieved = per[f"{dom}_GBps"]
+    line = {
+        "metric": "dispatch+combine GB/s of one rank's plan->dispatch->combine chain (plan us reported beside)",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "config 1: single-rank dispatch+combine, S=4096 H=7168 K=8 E=256 R=8 "
+                               "token_padding=128, plan->dispatch->combine under one HIP graph",
+                   "maxvio": round(ch.maxvio, 3), "seed": args.seed, "rank": rank},
+        "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
+        "graph_ms_per_step_events": ev_ms,
+        "plan_us": per["plan_us"], "dispatch_us": per["dispatch_us"], "combine_us": per["combine_us"],
+        "dispatch_GBps": per["dispatch_GBps"], "combine_GBps": per["combine_GBps"],
+        "dispatch_pct_hbm_peak": 100.0 * per["dispatch_GBps"] / HBM_PEAK_GBPS,
+        "combine_pct_hbm_peak": 100.0 * per["combine_GBps"] / HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": f"{dom}_kernel", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "algorithmic_bytes": by, "traffic": MEASURED_TRAFFIC_BYTES[dom]},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(ch)
+    ch.destroy()
+    torch.cuda.empty_cache()
+    if args.full:
+        sweep = {}
+        for shape in ((4096, 7168, 256), (8192, 4096, 128)):
+            for mv in (0.0, 0.5, 1.0, 2.0, 4.0):
+                c2 = Chain(shape[0], shape[1], K, shape[2], R, tp, rank, mv, args.seed)
+                w2, e2, p2 = measure_chain(c2, args.steps, args.warmup)
+                sweep[f"S{shape[0]}_H{shape[1]}_E{shape[2]}_maxvio{mv}"] = {
+                    "maxvio": round(c2.maxvio, 3), "chain_us": w2 * 1e3, "plan_us": p2["plan_us"],
+                    "dispatch_us": p2["dispatch_us"], "combine_us": p2["combine_us"]}
+                c2.destroy()
+                torch.cuda.empty_cache()
+        line["maxvio_sweep"] = sweep
+        line["weights"] = bench_weights(args.seed, max(5, args.steps // 2))
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -158,10 +158,21 @@ def test_world_dispatch_combine_matches_oracle(cuda, case):
             assert torch.equal(out_w.cpu().view(torch.int32), want_w.view(torch.int32))
             # the gathered weights are the ones this rank scattered
             assert torch.equal(out_w.cpu().view(torch.int32), wts[r].view(torch.int32))
-            # within 1 ulp (+0.5) of the single-rounding fp32 K-sum
-            ref_all, _ = oo.combine(expert_out, None, dst_r, K, mode="all")
-            err = (out.cpu().float() - ref_all.float()).abs() / oo.bf16_ulp(ref_all)
-            assert float(err.max()) <= 1.5, (mode, r, float(err.max()))
+    # Tolerance of the reference's own test (tests/test_combine.py:202-211):
+    # within 1 bf16 ulp (+0.5 slack) of the single-rounding fp32 K-sum, on
+    # same-sign data (with cancellation the group rounding of the reference
+    # pipeline is not small against the final result's ulp).
+    pos = (expert_out.float().abs() + 0.25).to(torch.bfloat16)
+    world.hidden_buf.copy_(pos.view(R * NvS, H))
+    for r in range(R):
+        dst_r = torch.from_numpy(plans[r].dst)
+        ref_all, _ = oo.combine(pos, None, dst_r, K, mode="all")
+        out = torch.empty(S, H, dtype=torch.bfloat16, device=cuda)
+        launch_combine(bufs[r]._require_ctx(), out, gplans[r].dst, None, mode="two_level")
+        torch.cuda.synchronize()
+        err = (out.cpu().float() - ref_all.float()).abs() / oo.bf16_ulp(ref_all)
+        assert float(err.max()) <= 1.5, (r, float(err.max()))
+    world.hidden_buf.copy_(expert_out.view(R * NvS, H))
     # reference pipeline: prologue on every rank, then primaries-only combine
     pro_ref = expert_out.clone()
     for r in range(R):
