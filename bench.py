@@ -39,6 +39,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--full", action="store_true", help="also sweep maxvio, 2nd shape, prefetch, grad reduce")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--profile-kernels", action="store_true",
+                    help="for rocprofv3: a few plain launches of each kernel and of a 512 MiB "
+                         "torch copy (the known-size kernel counters are scaled by); no JSON")
     ap.add_argument("--maxvio", type=float, default=1.0)
     ap.add_argument("--seed", type=int, default=2024)
     return ap.parse_args()
@@ -253,6 +256,16 @@ def main():
     torch.cuda.set_device(0)
     S, H, K, E, R, tp, rank = 4096, 7168, 8, 256, 8, 128, 0
     ch = Chain(S, H, K, E, R, tp, rank, args.maxvio, args.seed)
+    if args.profile_kernels:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda").view(torch.float32)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)            # reads 512 MiB, writes 512 MiB
+            ch.plan_fn(); ch.dispatch_fn(0); ch.combine_fn(0)
+            torch.cuda.synchronize()
+        print("profile-kernels: 3 x (copy 512MiB, plan, dispatch, combine) launched", file=sys.stderr)
+        ch.destroy()
+        return
     wall_ms, ev_ms, per = measure_chain(ch, args.steps, args.warmup)
     by = ch.bytes_one_way()
     value = 2 * by / (wall_ms * 1e-3) / 1e9

@@ -16,7 +16,7 @@ struct CombineArgs {
   uint16_t* out;
   float* out_sk;
   int64_t shard_stride_rows, wslot_stride;
-  int S, H, K, R, NvS, mode;
+  int S, H, K, R, NvS, mode, parts;
 };
 
 __device__ __forceinline__ void acc8(float* acc, mep_u4 v) {
@@ -27,11 +27,17 @@ __device__ __forceinline__ void acc8(float* acc, mep_u4 v) {
   }
 }
 
-// CH: 16-byte chunks a lane keeps in flight per row (unrolled).
-template <int CH>
+// A wave sums CH consecutive 1-KiB chunks (64 lanes x 16 bytes) of one token's
+// rows; a token takes `parts` waves.  EXACT: the row is a whole number of such
+// wave tiles, so no bounds checks.  All CH loads of a row are issued before
+// they are consumed: with K rows that keeps CH x 1 KiB per wave in flight.
+// TWO: the two-level mode (it carries a second accumulator set).
+template <int CH, bool EXACT, bool TWO>
 __global__ __launch_bounds__(kBlock) void combine_kernel(CombineArgs a) {
   const int lane = threadIdx.x & 63;
-  const int s = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int gw = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int s = gw / a.parts;
+  const int part = gw - s * a.parts;
   if (s >= a.S) return;
   const int K = a.K;
   const size_t row_bytes = (size_t)a.H * 2;
@@ -41,108 +47,111 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(CombineArgs a) {
   const int drank = raw / a.NvS;
   const int loff = raw - drank * a.NvS;
   const bool valid = lane < K && drank < a.R;
-  if (a.out_sk && lane < K)
+  if (a.out_sk && part == 0 && lane < K)
     a.out_sk[(size_t)s * K + lane] = valid ? a.wslots[(size_t)drank * a.wslot_stride + loff] : 0.0f;
   const uint64_t off = ((uint64_t)drank * (uint64_t)a.shard_stride_rows + (uint64_t)loff) * row_bytes;
   const uint32_t off_lo = (uint32_t)off, off_hi = (uint32_t)(off >> 32);
   const bool primary = valid && dv >= 0;
   const uint64_t prim_mask = __ballot(primary);
   const uint64_t valid_mask = __ballot(valid);
-  const char* base = (const char*)a.shards;
-  char* orow = (char*)a.out + (size_t)s * row_bytes;
   const int nvec = a.H / 8;
+  const int c0 = part * CH * 64 + lane;  // this lane's first 16-byte vector
+  const char* base = (const char*)a.shards + (size_t)c0 * 16;
+  char* orow = (char*)a.out + (size_t)s * row_bytes + (size_t)c0 * 16;
 
-  if (a.mode != MEP_COMBINE_TWO_LEVEL) {
-    const uint64_t sel = a.mode == MEP_COMBINE_ALL ? valid_mask : prim_mask;
-    for (int c0 = 0; c0 < nvec; c0 += CH * 64) {
-      float acc[CH][8];
+  float acc[CH][8];
 #pragma unroll
-      for (int i = 0; i < CH; ++i)
+  for (int i = 0; i < CH; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = 0.0f;
-      uint64_t t = sel;
-      while (t) {
-        const int k = __ffsll((unsigned long long)t) - 1;
-        t &= t - 1;
-        const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(off_hi, k) << 32) |
-                           (uint32_t)__builtin_amdgcn_readlane(off_lo, k);
-        const char* row = base + o;
-        mep_u4 v[CH];
+    for (int j = 0; j < 8; ++j) acc[i][j] = 0.0f;
+
+  auto row_of = [&](int k) -> const char* {
+    const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(off_hi, k) << 32) |
+                       (uint32_t)__builtin_amdgcn_readlane(off_lo, k);
+    return base + o;
+  };
+  auto load_row = [&](const char* row, mep_u4* v) {
 #pragma unroll
-        for (int i = 0; i < CH; ++i) {
-          const int c = c0 + i * 64 + lane;
-          v[i] = mep_u4{0u, 0u, 0u, 0u};
-          if (c < nvec) v[i] = mep_ld16_stream(row + (size_t)c * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < CH; ++i) acc8(acc[i], v[i]);
-      }
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        const int c = c0 + i * 64 + lane;
-        if (c < nvec) {
-          mep_u4 o;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) o[j] = mep_pack_bf16(acc[i][2 * j], acc[i][2 * j + 1]);
-          mep_st16_stream(orow + (size_t)c * 16, o);
-        }
-      }
+    for (int i = 0; i < CH; ++i) {
+      v[i] = mep_u4{0u, 0u, 0u, 0u};
+      if (EXACT || c0 + i * 64 < nvec) v[i] = mep_ld16_stream(row + (size_t)i * 1024);
     }
-    return;
-  }
+  };
 
-  // two-level: per destination-rank group (primary, then its duplicates in
-  // ascending k) an fp32 sum rounded to bf16; then the sum of the groups.
-  // members of the group led by entry k: later non-primary entries on the
-  // same destination rank.
-  uint64_t members = 0;  // lane k keeps the member mask of its own group
-  {
+  if (!TWO) {
+    uint64_t t = a.mode == MEP_COMBINE_ALL ? valid_mask : prim_mask;
+    while (t) {
+      const int k = __ffsll((unsigned long long)t) - 1;
+      t &= t - 1;
+      mep_u4 v[CH];
+      load_row(row_of(k), v);
+#pragma unroll
+      for (int i = 0; i < CH; ++i) acc8(acc[i], v[i]);
+    }
+  } else {
+    // Per destination-rank group (its primary, then its duplicates in
+    // ascending k) an fp32 sum rounded to bf16; then the sum of the groups in
+    // the order of their primaries.  Lane k keeps the member mask of the
+    // group it leads: later non-primary entries on the same rank.
+    uint64_t members = 0;
     for (int k = 0; k < K; ++k) {
       const int dk = __builtin_amdgcn_readlane(drank, k);
       const uint64_t m = __ballot(valid && !primary && drank == dk && lane > k);
       if (lane == k) members = m;
     }
-  }
-  const uint32_t mem_lo = (uint32_t)members, mem_hi = (uint32_t)(members >> 32);
-  for (int c = lane; c < nvec + lane; c += 64) {  // uniform trip count across the wave
-    const bool in = c < nvec;
-    float acc[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    const uint32_t mem_lo = (uint32_t)members, mem_hi = (uint32_t)(members >> 32);
     uint64_t t = prim_mask;
     while (t) {
       const int k = __ffsll((unsigned long long)t) - 1;
       t &= t - 1;
-      const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(off_hi, k) << 32) |
-                         (uint32_t)__builtin_amdgcn_readlane(off_lo, k);
       uint64_t mem = ((uint64_t)__builtin_amdgcn_readlane(mem_hi, k) << 32) |
                      (uint32_t)__builtin_amdgcn_readlane(mem_lo, k);
-      float grp[8];
+      mep_u4 v[CH];
+      load_row(row_of(k), v);
+      if (mem == 0) {  // a group of one: bf16(row) is the row itself
 #pragma unroll
-      for (int j = 0; j < 8; ++j) grp[j] = 0.0f;
-      mep_u4 v = mep_u4{0u, 0u, 0u, 0u};
-      if (in) v = mep_ld16_stream(base + o + (size_t)c * 16);
-      acc8(grp, v);
-      const bool rounded = mem != 0;
+        for (int i = 0; i < CH; ++i) acc8(acc[i], v[i]);
+        continue;
+      }
+      float grp[CH][8];
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) grp[i][j] = 0.0f;
+        acc8(grp[i], v[i]);
+      }
       while (mem) {
         const int j2 = __ffsll((unsigned long long)mem) - 1;
         mem &= mem - 1;
-        const uint64_t o2 = ((uint64_t)__builtin_amdgcn_readlane(off_hi, j2) << 32) |
-                            (uint32_t)__builtin_amdgcn_readlane(off_lo, j2);
-        mep_u4 v2 = mep_u4{0u, 0u, 0u, 0u};
-        if (in) v2 = mep_ld16_stream(base + o2 + (size_t)c * 16);
-        acc8(grp, v2);
+        load_row(row_of(j2), v);
+#pragma unroll
+        for (int i = 0; i < CH; ++i) acc8(grp[i], v[i]);
       }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] += rounded ? mep_round_bf16(grp[j]) : grp[j];
-    }
-    if (in) {
-      mep_u4 o;
+      for (int i = 0; i < CH; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o[j] = mep_pack_bf16(acc[2 * j], acc[2 * j + 1]);
-      mep_st16_stream(orow + (size_t)c * 16, o);
+        for (int j = 0; j < 8; ++j) acc[i][j] += mep_round_bf16(grp[i][j]);
     }
   }
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    if (EXACT || c0 + i * 64 < nvec) {
+      mep_u4 o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = mep_pack_bf16(acc[i][2 * j], acc[i][2 * j + 1]);
+      mep_st16_stream(orow + (size_t)i * 1024, o);
+    }
+  }
+}
+
+template <int CH, bool EXACT, bool TWO>
+void launch_combine(const CombineArgs& a0, hipStream_t st) {
+  CombineArgs a = a0;
+  const int nvec = a.H / 8;
+  a.parts = (nvec + CH * 64 - 1) / (CH * 64);
+  const int64_t waves = (int64_t)a.S * a.parts;
+  dim3 grid((unsigned)((waves + kWavesPerBlock - 1) / kWavesPerBlock));
+  hipLaunchKernelGGL((combine_kernel<CH, EXACT, TWO>), grid, dim3(kBlock), 0, st, a);
 }
 
 }  // namespace
@@ -163,7 +172,20 @@ extern "C" int mep_combine(const void* shards, int64_t shard_stride_rows, const 
   a.out = (uint16_t*)out_SH; a.out_sk = out_SK;
   a.shard_stride_rows = shard_stride_rows; a.wslot_stride = wslot_stride;
   a.S = S; a.H = H; a.K = K; a.R = R; a.NvS = NvS; a.mode = mode;
-  dim3 grid((S + kWavesPerBlock - 1) / kWavesPerBlock);
-  hipLaunchKernelGGL(combine_kernel<2>, grid, dim3(kBlock), 0, (hipStream_t)stream, a);
+  a.parts = 1;
+  hipStream_t st = (hipStream_t)stream;
+  const int nvec = H / 8;
+  // widest wave tile that divides the row; the two-level mode takes tiles of
+  // half the width
+  if (mode == MEP_COMBINE_TWO_LEVEL) {
+    if (nvec % (7 * 64) == 0) launch_combine<7, true, true>(a, st);
+    else if (nvec % (4 * 64) == 0) launch_combine<4, true, true>(a, st);
+    else launch_combine<2, false, true>(a, st);
+  } else {
+    if (nvec % (14 * 64) == 0) launch_combine<14, true, false>(a, st);
+    else if (nvec % (8 * 64) == 0) launch_combine<8, true, false>(a, st);
+    else if (nvec % (4 * 64) == 0) launch_combine<4, true, false>(a, st);
+    else launch_combine<2, false, false>(a, st);
+  }
   return mep_launch_status();
 }

@@ -1,7 +1,9 @@
 // Dispatch side of the hot path for gfx950: fused permute (one wave per token
-// row, the row is read once into registers and streamed to every destination
-// slot), weight scatter, padding zero-fill, duplicate-group builder and the
-// destination-side duplicate expansion.
+// row; the row is read once into registers with ordinary loads -- it was just
+// produced and is often still cached -- and streamed to every destination slot
+// with nontemporal stores, which leave the cached inputs alone), weight
+// scatter, padding zero-fill, duplicate-group builder and the destination-side
+// duplicate expansion.
 #include "mep_common.h"
 
 namespace {
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
     if (NV > 0) {
       mep_u4 v[NV > 0 ? NV : 1];
 #pragma unroll
-      for (int i = 0; i < NV; ++i) v[i] = mep_ld16_stream(src + ((size_t)i * 64 + lane) * 16);
+      for (int i = 0; i < NV; ++i) v[i] = mep_ld16(src + ((size_t)i * 64 + lane) * 16);
       while (todo) {
         const int k = __ffsll((unsigned long long)todo) - 1;
         todo &= todo - 1;
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int c = c0 + i * 64 + lane;
-          if (c < nvec) v[i] = mep_ld16_stream(src + (size_t)c * 16);
+          if (c < nvec) v[i] = mep_ld16(src + (size_t)c * 16);
         }
         uint64_t t = todo;
         while (t) {

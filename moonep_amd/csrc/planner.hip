@@ -61,8 +61,8 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   int* s_cd = s_ce + NT;         // [NT] destination rank of each entry
   int* tbl = kLdsTables ? (s_cd + NT)
                         : a.scratch + (size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 2 * E * R;
-  int* alloc = tbl;            // [E,R] tokens of e on d, later its prefix over d
-  int* base = tbl + E * R;     // [E,R] dst = base[e,d] + global index of the entry
+  int* alloc = tbl;            // [E,R] tokens of expert e landing on rank d
+  int* base = tbl + E * R;     // [E,R] first slot of e on d, as an encoded dst
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -95,23 +95,20 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   // Each receiver is filled exactly once (to capacity), so z[h][u] of the
   // reference (tests/planning_reference.py:85-96) is stored per receiver.
   if (wave == 0) {
-    int b0 = lane < R ? s_gt[lane] - CAP : 0;
-    int b1 = lane + 64 < R ? s_gt[lane + 64] - CAP : 0;
-    const bool v0 = lane < R, v1 = lane + 64 < R;
+    for (int k = lane; k < R; k += 64) s_bal[k] = s_gt[k] - CAP;
+    mep_wave_sync();
     for (int it = 0; it < R; ++it) {
-      // candidate of this lane for max (first index wins ties) and min
-      int mx = v0 ? b0 : INT32_MIN, mxi = lane;
-      if (v1 && b1 > mx) { mx = b1; mxi = lane + 64; }
-      int mn = v0 ? b0 : INT32_MAX, mni = lane;
-      if (v1 && b1 < mn) { mn = b1; mni = lane + 64; }
-      int hv, h, uv, u;
-      mep_wave_argmax_first(mx, mxi, hv, h);
-      mep_wave_argmin_first(mn, mni, uv, u);
+      // all lanes read the same words (LDS broadcast): no cross-lane reduction
+      int hv = INT32_MIN, h = 0, uv = INT32_MAX, u = 0;
+      for (int r = 0; r < R; ++r) {
+        const int b = s_bal[r];
+        if (b > hv) { hv = b; h = r; }   // first index wins ties
+        if (b < uv) { uv = b; u = r; }
+      }
       if (hv <= 0 || uv >= 0) break;
-      const int move = -uv;
-      if (lane == (h & 63)) { if (h < 64) b0 -= move; else b1 -= move; }
-      if (lane == (u & 63)) { if (u < 64) b0 = 0; else b1 = 0; }
-      if (lane == 0) { s_from[u] = h; s_quota[u] = move; }
+      mep_wave_sync();
+      if (lane == 0) { s_bal[h] = hv + uv; s_bal[u] = 0; s_from[u] = h; s_quota[u] = -uv; }
+      mep_wave_sync();
     }
   }
   __syncthreads();
@@ -120,13 +117,11 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   for (int h = wave; h < R; h += NW) {
     const int es = h * epn;
     for (int it = 0; it < R + epn; ++it) {
-      int q = INT32_MIN, qi = INT32_MAX;
-      for (int d = lane; d < R; d += 64) {
-        int v = (s_from[d] == h) ? s_quota[d] : 0;
-        if (v > q) { q = v; qi = d; }
+      int quota = 0, d = 0;
+      for (int r = 0; r < R; ++r) {
+        const int v = (s_from[r] == h) ? s_quota[r] : 0;
+        if (v > quota) { quota = v; d = r; }
       }
-      int quota, d;
-      mep_wave_argmax_first(q, qi, quota, d);
       if (quota <= 0) break;
       int rm = INT32_MIN, ri = INT32_MAX;
       for (int le = lane; le < epn; le += 64) {
@@ -200,17 +195,6 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
     }
   }
 
-  // ---- prefix over destinations; fold it into the slot base --------------
-  for (int e = tid; e < E; e += NT) {
-    int run = 0;
-    for (int d = 0; d < R; ++d) {
-      const int v = alloc[e * R + d];
-      base[e * R + d] -= run;
-      run += v;
-      alloc[e * R + d] = run;
-    }
-  }
-
   // ---- my slice of the rank's entries -------------------------------------
   const int* topk = a.topk + (size_t)blockIdx.y * N;
   int* dst = a.dst + (size_t)blockIdx.y * N;
@@ -219,29 +203,52 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   const int e0 = t0 * K;
   const int n = (t1 - t0) * K;  // <= NT
 
-  // entries before my slice, per expert
-  for (int i = tid; i < e0; i += NT) {
-    const int e = topk[i];
-    if ((unsigned)e < (unsigned)E) atomicAdd(&s_hist[e], 1);
+  // entries before my slice, per expert (16-byte loads, four in flight)
+  {
+    int done = 0;
+    if ((((uintptr_t)topk) & 15) == 0) {
+      const int nv = e0 >> 2;
+      const int4* t4 = (const int4*)topk;
+      for (int i = tid; i < nv; i += 4 * NT) {
+        int4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (i + u * NT < nv) v[u] = t4[i + u * NT];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (i + u * NT < nv) {
+            if ((unsigned)v[u].x < (unsigned)E) atomicAdd(&s_hist[v[u].x], 1);
+            if ((unsigned)v[u].y < (unsigned)E) atomicAdd(&s_hist[v[u].y], 1);
+            if ((unsigned)v[u].z < (unsigned)E) atomicAdd(&s_hist[v[u].z], 1);
+            if ((unsigned)v[u].w < (unsigned)E) atomicAdd(&s_hist[v[u].w], 1);
+          }
+      }
+      done = nv << 2;
+    }
+    for (int i = done + tid; i < e0; i += NT) {
+      const int ee = topk[i];
+      if ((unsigned)ee < (unsigned)E) atomicAdd(&s_hist[ee], 1);
+    }
   }
   int e = -1;
   if (tid < n) {
     e = topk[e0 + tid];
     if ((unsigned)e >= (unsigned)E) e = -1;  // invalid id: slot 0, never out of bounds
   }
-  // position among equal experts inside my wave
+  // lanes of my wave holding the same expert: one ballot per key bit
   int pos = 0;
   {
-    uint64_t todo = __ballot(e >= 0);
-    while (todo) {
-      const int leader = __ffsll((unsigned long long)todo) - 1;
-      const int ev = __builtin_amdgcn_readlane(e, leader);
-      const uint64_t m = __ballot(e == ev);
-      if (e == ev) {
-        pos = __popcll(m & mep_lanes_lt());
-        if (pos == 0) atomicAdd(&s_wcnt[e * W4 + (wave >> 2)], __popcll(m) << (8 * (wave & 3)));
-      }
-      todo &= ~m;
+    uint64_t same = __ballot(e >= 0);
+    const int nbits = 32 - __clz(E - 1 > 0 ? E - 1 : 1);
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = (e >> b) & 1;
+      const uint64_t bb = __ballot(bit);
+      same &= bit ? bb : ~bb;
+    }
+    if (e >= 0) {
+      pos = __popcll(same & mep_lanes_lt());
+      if (pos == 0)
+        atomicAdd(&s_wcnt[e * W4 + (wave >> 2)], __popcll(same) << (8 * (wave & 3)));
     }
   }
   __syncthreads();
@@ -253,8 +260,14 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       for (int b = 0; b < 4; ++b)
         if (w4 * 4 + b < wave) before += (word >> (8 * b)) & 0xffu;
     }
-    const int g = s_prev[e] + s_hist[e] + before + pos;
-    while (dest < R - 1 && alloc[e * R + dest] <= g) ++dest;
+    // entries of expert e are numbered over (source rank, flat index) and cut
+    // into the destinations' allocations in rank order
+    int g = s_prev[e] + s_hist[e] + before + pos;
+    for (; dest < R - 1; ++dest) {
+      const int c = alloc[e * R + dest];
+      if (g < c) break;
+      g -= c;
+    }
     dv = base[e * R + dest] + g;
   }
   s_cd[tid] = dest;
