@@ -79,10 +79,15 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   __syncthreads();
   for (int e = tid; e < E; e += NT) {
     int c = 0, p = 0;
-    for (int r = 0; r < R; ++r) {
-      int v = a.tpe[r * E + e];
-      if (r < rank) p += v;
-      c += v;
+    for (int r0 = 0; r0 < R; r0 += 8) {  // eight independent loads in flight
+      int v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = r0 + j < R ? a.tpe[(r0 + j) * E + e] : 0;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (r0 + j < rank) p += v[j];
+        c += v[j];
+      }
     }
     s_cnt[e] = c; s_prev[e] = p; s_rem[e] = c;
     const int home = e / epn;
