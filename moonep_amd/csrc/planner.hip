@@ -96,41 +96,139 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   }
   __syncthreads();
 
-  // ---- receivers and quotas: one wave, balances in registers -------------
+  // ---- receivers and quotas (wave 0) | histogram of earlier entries -------
   // Each receiver is filled exactly once (to capacity), so z[h][u] of the
   // reference (tests/planning_reference.py:85-96) is stored per receiver.
+  // The upper half of the waves meanwhile counts, per expert, this rank's
+  // entries that precede the workgroup's slice: that needs nothing from the
+  // plan and hides behind the serial greedy loops.
+  const int* topk = a.topk + (size_t)blockIdx.y * N;
+  const int t0 = blockIdx.x * a.tok_per_wg;
+  const int t1 = min(t0 + a.tok_per_wg, a.S);
+  const int e0 = t0 * K;
+  const int n = (t1 - t0) * K;  // <= NT
   if (wave == 0) {
-    for (int k = lane; k < R; k += 64) s_bal[k] = s_gt[k] - CAP;
-    mep_wave_sync();
-    for (int it = 0; it < R; ++it) {
-      // all lanes read the same words (LDS broadcast): no cross-lane reduction
-      int hv = INT32_MIN, h = 0, uv = INT32_MAX, u = 0;
-      for (int r = 0; r < R; ++r) {
-        const int b = s_bal[r];
-        if (b > hv) { hv = b; h = r; }   // first index wins ties
-        if (b < uv) { uv = b; u = r; }
+    if (R <= 8) {
+      // every lane keeps all balances in registers: no cross-lane traffic
+      int bal[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) bal[r] = r < R ? s_gt[r] - CAP : 0;
+      for (int it = 0; it < R; ++it) {
+        int hv = INT32_MIN, h = 0, uv = INT32_MAX, u = 0;
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          if (r < R) {
+            if (bal[r] > hv) { hv = bal[r]; h = r; }  // first index wins ties
+            if (bal[r] < uv) { uv = bal[r]; u = r; }
+          }
+        if (hv <= 0 || uv >= 0) break;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          if (r == h) bal[r] = hv + uv;
+          if (r == u) bal[r] = 0;
+        }
+        if (lane == 0) { s_from[u] = h; s_quota[u] = -uv; }
       }
-      if (hv <= 0 || uv >= 0) break;
-      mep_wave_sync();
-      if (lane == 0) { s_bal[h] = hv + uv; s_bal[u] = 0; s_from[u] = h; s_quota[u] = -uv; }
-      mep_wave_sync();
+    } else {
+      int b0 = lane < R ? s_gt[lane] - CAP : 0;
+      int b1 = lane + 64 < R ? s_gt[lane + 64] - CAP : 0;
+      const bool v0 = lane < R, v1 = lane + 64 < R;
+      for (int it = 0; it < R; ++it) {
+        int mx = v0 ? b0 : INT32_MIN, mxi = lane;
+        if (v1 && b1 > mx) { mx = b1; mxi = lane + 64; }
+        int mn = v0 ? b0 : INT32_MAX, mni = lane;
+        if (v1 && b1 < mn) { mn = b1; mni = lane + 64; }
+        int hv, h, uv, u;
+        mep_wave_argmax_first(mx, mxi, hv, h);
+        mep_wave_argmin_first(mn, mni, uv, u);
+        if (hv <= 0 || uv >= 0) break;
+        const int move = -uv;
+        if (lane == (h & 63)) { if (h < 64) b0 -= move; else b1 -= move; }
+        if (lane == (u & 63)) { if (u < 64) b0 = 0; else b1 = 0; }
+        if (lane == 0) { s_from[u] = h; s_quota[u] = move; }
+      }
+    }
+  } else if (wave >= NW / 2) {
+    constexpr int HT = NT - (NW / 2) * 64;  // threads counting
+    const int ht = tid - (NW / 2) * 64;
+    int done = 0;
+    if ((((uintptr_t)topk) & 15) == 0) {  // 16-byte loads, four in flight
+      const int nv = e0 >> 2;
+      const int4* t4 = (const int4*)topk;
+      for (int i = ht; i < nv; i += 4 * HT) {
+        int4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (i + u * HT < nv) v[u] = t4[i + u * HT];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (i + u * HT < nv) {
+            if ((unsigned)v[u].x < (unsigned)E) atomicAdd(&s_hist[v[u].x], 1);
+            if ((unsigned)v[u].y < (unsigned)E) atomicAdd(&s_hist[v[u].y], 1);
+            if ((unsigned)v[u].z < (unsigned)E) atomicAdd(&s_hist[v[u].z], 1);
+            if ((unsigned)v[u].w < (unsigned)E) atomicAdd(&s_hist[v[u].w], 1);
+          }
+      }
+      done = nv << 2;
+    }
+    for (int i = done + ht; i < e0; i += HT) {
+      const int ee = topk[i];
+      if ((unsigned)ee < (unsigned)E) atomicAdd(&s_hist[ee], 1);
     }
   }
   __syncthreads();
 
   // ---- which tokens of which expert migrate: one wave per home group -----
+  // An (expert, receiver) pair is touched at most once (every step exhausts
+  // the expert or the receiver), so alloc[e][d] is a plain store and what
+  // stays home is written once at the end.
+  const bool packed_key = (int64_t)R * CAP < (1 << 25);  // count and lane fit one int
   for (int h = wave; h < R; h += NW) {
     const int es = h * epn;
-    for (int it = 0; it < R + epn; ++it) {
-      int quota = 0, d = 0;
-      for (int r = 0; r < R; ++r) {
-        const int v = (s_from[r] == h) ? s_quota[r] : 0;
-        if (v > quota) { quota = v; d = r; }
+    if (R <= 8 && epn <= 64) {
+      int q[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) q[r] = (r < R && s_from[r] == h) ? s_quota[r] : 0;
+      int rem = lane < epn ? s_rem[es + lane] : -1;
+      for (int it = 0; it < R + epn; ++it) {
+        int quota = 0, d = 0;
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          if (q[r] > quota) { quota = q[r]; d = r; }
+        if (quota <= 0) break;
+        int best, le;
+        if (packed_key) {
+          const int m = mep_wave_max(rem < 0 ? INT32_MIN : (rem << 6) | (63 - lane));
+          best = m >> 6;
+          le = 63 - (m & 63);
+        } else {
+          mep_wave_argmax_first(rem, lane, best, le);
+        }
+        if (best <= 0) break;
+        const int take = best < quota ? best : quota;
+        if (lane == le) {
+          rem -= take;
+          alloc[(es + le) * R + d] = take;
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          if (r == d) q[r] -= take;
       }
+      if (lane < epn) alloc[(es + lane) * R + h] = rem;
+      continue;
+    }
+    for (int it = 0; it < R + epn; ++it) {
+      int q = INT32_MIN, qi = INT32_MAX;
+      for (int d = lane; d < R; d += 64) {
+        const int v = (s_from[d] == h) ? s_quota[d] : 0;
+        if (v > q) { q = v; qi = d; }
+      }
+      int quota, d;
+      mep_wave_argmax_first(q, qi, quota, d);
       if (quota <= 0) break;
       int rm = INT32_MIN, ri = INT32_MAX;
       for (int le = lane; le < epn; le += 64) {
-        int v = s_rem[es + le];
+        const int v = s_rem[es + le];
         if (v > rm) { rm = v; ri = le; }
       }
       int rem, le;
@@ -139,8 +237,8 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       const int take = rem < quota ? rem : quota;
       if (lane == 0) {
         const int e = es + le;
-        alloc[e * R + d] += take;
-        alloc[e * R + h] -= take;
+        alloc[e * R + d] = take;
+        alloc[e * R + h] = rem - take;
         s_rem[e] = rem - take;
         s_quota[d] = quota - take;
       }
@@ -201,40 +299,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   }
 
   // ---- my slice of the rank's entries -------------------------------------
-  const int* topk = a.topk + (size_t)blockIdx.y * N;
   int* dst = a.dst + (size_t)blockIdx.y * N;
-  const int t0 = blockIdx.x * a.tok_per_wg;
-  const int t1 = min(t0 + a.tok_per_wg, a.S);
-  const int e0 = t0 * K;
-  const int n = (t1 - t0) * K;  // <= NT
-
-  // entries before my slice, per expert (16-byte loads, four in flight)
-  {
-    int done = 0;
-    if ((((uintptr_t)topk) & 15) == 0) {
-      const int nv = e0 >> 2;
-      const int4* t4 = (const int4*)topk;
-      for (int i = tid; i < nv; i += 4 * NT) {
-        int4 v[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (i + u * NT < nv) v[u] = t4[i + u * NT];
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (i + u * NT < nv) {
-            if ((unsigned)v[u].x < (unsigned)E) atomicAdd(&s_hist[v[u].x], 1);
-            if ((unsigned)v[u].y < (unsigned)E) atomicAdd(&s_hist[v[u].y], 1);
-            if ((unsigned)v[u].z < (unsigned)E) atomicAdd(&s_hist[v[u].z], 1);
-            if ((unsigned)v[u].w < (unsigned)E) atomicAdd(&s_hist[v[u].w], 1);
-          }
-      }
-      done = nv << 2;
-    }
-    for (int i = done + tid; i < e0; i += NT) {
-      const int ee = topk[i];
-      if ((unsigned)ee < (unsigned)E) atomicAdd(&s_hist[ee], 1);
-    }
-  }
   int e = -1;
   if (tid < n) {
     e = topk[e0 + tid];
