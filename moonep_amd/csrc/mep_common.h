@@ -78,6 +78,26 @@ __device__ __forceinline__ int mep_wave_min(int v) {
   return __builtin_amdgcn_readlane(v, 63);
 }
 
+// The same over the first 16 lanes only (one DPP row): for tables of at most
+// 16 entries; lanes past the table must hold the identity.
+__device__ __forceinline__ int mep_row_max(int v) {
+  const int id = INT32_MIN;
+  MEP_DPP_STEP(mep_imax, v, id, 0x111, 0xf);
+  MEP_DPP_STEP(mep_imax, v, id, 0x112, 0xf);
+  MEP_DPP_STEP(mep_imax, v, id, 0x114, 0xf);
+  MEP_DPP_STEP(mep_imax, v, id, 0x118, 0xf);
+  return __builtin_amdgcn_readlane(v, 15);
+}
+
+__device__ __forceinline__ int mep_row_min(int v) {
+  const int id = INT32_MAX;
+  MEP_DPP_STEP(mep_imin, v, id, 0x111, 0xf);
+  MEP_DPP_STEP(mep_imin, v, id, 0x112, 0xf);
+  MEP_DPP_STEP(mep_imin, v, id, 0x114, 0xf);
+  MEP_DPP_STEP(mep_imin, v, id, 0x118, 0xf);
+  return __builtin_amdgcn_readlane(v, 15);
+}
+
 // Inclusive prefix sum across the wave (lane i gets v_0 + ... + v_i).
 __device__ __forceinline__ int mep_wave_incl_scan(int v) {
   MEP_DPP_STEP(mep_iadd, v, 0, 0x111, 0xf);

@@ -107,46 +107,37 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   const int t1 = min(t0 + a.tok_per_wg, a.S);
   const int e0 = t0 * K;
   const int n = (t1 - t0) * K;  // <= NT
+  // (value, index) pairs travel through one reduction as value*128 + index
+  // code whenever the counts leave 7 bits of room
+  const bool packed_key = (int64_t)R * CAP < (1 << 24);
   if (wave == 0) {
-    if (R <= 8) {
-      // every lane keeps all balances in registers: no cross-lane traffic
-      int bal[8];
-#pragma unroll
-      for (int r = 0; r < 8; ++r) bal[r] = r < R ? s_gt[r] - CAP : 0;
-      for (int it = 0; it < R; ++it) {
-        int hv = INT32_MIN, h = 0, uv = INT32_MAX, u = 0;
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-          if (r < R) {
-            if (bal[r] > hv) { hv = bal[r]; h = r; }  // first index wins ties
-            if (bal[r] < uv) { uv = bal[r]; u = r; }
-          }
-        if (hv <= 0 || uv >= 0) break;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          if (r == h) bal[r] = hv + uv;
-          if (r == u) bal[r] = 0;
-        }
-        if (lane == 0) { s_from[u] = h; s_quota[u] = -uv; }
-      }
-    } else {
-      int b0 = lane < R ? s_gt[lane] - CAP : 0;
-      int b1 = lane + 64 < R ? s_gt[lane + 64] - CAP : 0;
-      const bool v0 = lane < R, v1 = lane + 64 < R;
-      for (int it = 0; it < R; ++it) {
+    // lane r keeps the balance of rank r (and of rank r + 64)
+    int b0 = lane < R ? s_gt[lane] - CAP : 0;
+    int b1 = lane + 64 < R ? s_gt[lane + 64] - CAP : 0;
+    const bool v0 = lane < R, v1 = lane + 64 < R;
+    for (int it = 0; it < R; ++it) {
+      int hv, h, uv, u;
+      if (packed_key) {
+        int kx = v0 ? b0 * 128 + (127 - lane) : INT32_MIN;  // max: first index wins ties
+        int kn = v0 ? b0 * 128 + lane : INT32_MAX;          // min: first index wins ties
+        if (v1) { kx = mep_imax(kx, b1 * 128 + (63 - lane)); kn = mep_imin(kn, b1 * 128 + lane + 64); }
+        kx = R <= 16 ? mep_row_max(kx) : mep_wave_max(kx);
+        kn = R <= 16 ? mep_row_min(kn) : mep_wave_min(kn);
+        hv = kx >> 7; h = 127 - (kx & 127);
+        uv = kn >> 7; u = kn & 127;
+      } else {
         int mx = v0 ? b0 : INT32_MIN, mxi = lane;
         if (v1 && b1 > mx) { mx = b1; mxi = lane + 64; }
         int mn = v0 ? b0 : INT32_MAX, mni = lane;
         if (v1 && b1 < mn) { mn = b1; mni = lane + 64; }
-        int hv, h, uv, u;
         mep_wave_argmax_first(mx, mxi, hv, h);
         mep_wave_argmin_first(mn, mni, uv, u);
-        if (hv <= 0 || uv >= 0) break;
-        const int move = -uv;
-        if (lane == (h & 63)) { if (h < 64) b0 -= move; else b1 -= move; }
-        if (lane == (u & 63)) { if (u < 64) b0 = 0; else b1 = 0; }
-        if (lane == 0) { s_from[u] = h; s_quota[u] = move; }
       }
+      if (hv <= 0 || uv >= 0) break;
+      const int move = -uv;
+      if (lane == (h & 63)) { if (h < 64) b0 -= move; else b1 -= move; }
+      if (lane == (u & 63)) { if (u < 64) b0 = 0; else b1 = 0; }
+      if (lane == 0) { s_from[u] = h; s_quota[u] = move; }
     }
   } else if (wave >= NW / 2) {
     constexpr int HT = NT - (NW / 2) * 64;  // threads counting
@@ -182,37 +173,28 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   // An (expert, receiver) pair is touched at most once (every step exhausts
   // the expert or the receiver), so alloc[e][d] is a plain store and what
   // stays home is written once at the end.
-  const bool packed_key = (int64_t)R * CAP < (1 << 25);  // count and lane fit one int
   for (int h = wave; h < R; h += NW) {
     const int es = h * epn;
-    if (R <= 8 && epn <= 64) {
-      int q[8];
-#pragma unroll
-      for (int r = 0; r < 8; ++r) q[r] = (r < R && s_from[r] == h) ? s_quota[r] : 0;
+    if (packed_key && R <= 64 && epn <= 64) {
+      // lane r keeps the open quota of receiver r, lane le what is left of
+      // the home's expert le
+      int q = (lane < R && s_from[lane] == h) ? s_quota[lane] : 0;
       int rem = lane < epn ? s_rem[es + lane] : -1;
       for (int it = 0; it < R + epn; ++it) {
-        int quota = 0, d = 0;
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-          if (q[r] > quota) { quota = q[r]; d = r; }
-        if (quota <= 0) break;
-        int best, le;
-        if (packed_key) {
-          const int m = mep_wave_max(rem < 0 ? INT32_MIN : (rem << 6) | (63 - lane));
-          best = m >> 6;
-          le = 63 - (m & 63);
-        } else {
-          mep_wave_argmax_first(rem, lane, best, le);
-        }
+        int kq = q > 0 ? q * 128 + (127 - lane) : INT32_MIN;
+        kq = R <= 16 ? mep_row_max(kq) : mep_wave_max(kq);
+        if (kq < 0) break;  // no open quota
+        const int quota = kq >> 7, d = 127 - (kq & 127);
+        int kr = rem >= 0 ? rem * 64 + (63 - lane) : INT32_MIN;
+        kr = epn <= 16 ? mep_row_max(kr) : mep_wave_max(kr);
+        const int best = kr >> 6, le = 63 - (kr & 63);
         if (best <= 0) break;
         const int take = best < quota ? best : quota;
         if (lane == le) {
           rem -= take;
           alloc[(es + le) * R + d] = take;
         }
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-          if (r == d) q[r] -= take;
+        if (lane == d) q -= take;
       }
       if (lane < epn) alloc[(es + lane) * R + h] = rem;
       continue;

@@ -89,3 +89,37 @@ def test_planner_matches_oracle_at_headline_shapes(cuda, S, H, K, E, R, mv):
     assert np.array_equal(plan.remote_stats.cpu().numpy(), plans[3].remote_stats)
     buf.destroy()
     buf3.destroy()
+
+
+@pytest.mark.parametrize("R,epn,S,K,tp,sigma", [
+    (16, 4, 64, 4, 16, 1.0),      # one DPP row of balances
+    (24, 3, 48, 6, 8, 2.0),       # full-wave reductions
+    (70, 2, 35, 4, 4, 1.5),       # ranks beyond lane 63
+    (128, 1, 64, 2, 8, 1.0),      # the encoding's rank limit
+    (12, 70, 96, 5, 32, 1.0),     # more than 64 experts per rank
+    (8, 8, 262144, 8, 128, 1.0),  # counts too large for packed (value, index) keys
+])
+def test_planner_wide_groups_match_oracle(cuda, R, epn, S, K, tp, sigma):
+    """Shapes outside the golden table (R > 8, large counts): the CPU oracle,
+    itself pinned by the golden vectors, is the reference."""
+    E = R * epn
+    if S >= 100000:
+        g = torch.Generator().manual_seed(5)
+        pop = torch.exp(torch.normal(0.0, sigma, (E,), generator=g))
+        topk = torch.multinomial(pop.expand(R * S, E), K, replacement=False, generator=g)
+        topk = topk.to(torch.int32).reshape(R, S, K)
+    else:
+        topk = torch.stack([routing.popularity_biased(S, K, E, R, r, sigma, seed=31) for r in range(R)])
+    tpe = routing.tokens_per_expert(topk, E)
+    print(f"R={R} epn={epn} S={S} K={K} tp={tp}", flush=True)
+    gp, plans, dst_all_ref = oracle_world_plan(topk.numpy(), tpe.numpy(), tp)
+    buf = Buffer(S, 16, K, E, R, token_padding=tp, rank=0)
+    dst_all, cu, etc, zfr, stats = launch_planning_all_ranks(buf._require_ctx(), topk.to(cuda),
+                                                             tpe.to(cuda))
+    torch.cuda.synchronize()
+    assert np.array_equal(dst_all.cpu().numpy(), dst_all_ref)
+    assert np.array_equal(cu.cpu().numpy(), gp.cu_seqlens)
+    assert np.array_equal(etc.cpu().numpy(), gp.experts_to_copy)
+    assert np.array_equal(zfr.cpu().numpy(), gp.zero_fill)
+    assert np.array_equal(stats.cpu().numpy(), gp.remote_stats)
+    buf.destroy()
