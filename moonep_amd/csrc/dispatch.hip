@@ -1,7 +1,7 @@
-// Dispatch side of the hot path for gfx950: fused permute (one wave per token
-// row; the row is read once into registers with ordinary loads -- it was just
-// produced and is often still cached -- and streamed to every destination slot
-// with nontemporal stores, which leave the cached inputs alone), weight
+// Dispatch side of the hot path for gfx950: fused permute (one wave per copy of
+// a token row; the row is read with ordinary loads -- it was just produced and
+// is shared by the token's K waves through the caches -- and streamed to its
+// slot with nontemporal stores, which leave the cached inputs alone), weight
 // scatter, padding zero-fill, duplicate-group builder and the destination-side
 // duplicate expansion.
 #include "mep_common.h"
@@ -23,8 +23,11 @@ struct DispatchArgs {
   unsigned flags;
 };
 
-// NV > 0: the row is exactly NV 16-byte vectors per lane and lives in
-// registers; NV == 0: any H % 8 == 0, strided loop.
+// One wave per (token, k) copy: it reads the token row (the K waves of a token
+// share it through the caches) and streams it to its slot.  Waves that issue
+// one row of stores each keep the HBM write path busier than one wave issuing
+// K rows.  NV > 0: the row is exactly NV 16-byte vectors per lane and passes
+// through registers in one go; NV == 0: any H % 8 == 0, strided loop.
 template <int NV>
 __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
   const int lane = threadIdx.x & 63;
@@ -32,58 +35,36 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
   const int H = a.H;
   const size_t row_bytes = (size_t)H * 2;
   if ((int)blockIdx.x < a.tok_blocks) {
-    const int s = blockIdx.x * kWavesPerBlock + wave;
-    if (s >= a.S) return;
-    const int K = a.K;
-    // lane k owns entry (s,k): decode, scatter its weight, publish its row address
-    int dv = 0;
-    if (lane < K) dv = a.dst[(size_t)s * K + lane];
+    const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;  // flat (token, k) index
+    if (gw >= (int64_t)a.S * a.K) return;
+    const int s = (int)(gw / a.K);
+    const int dv = a.dst[gw];
     const int raw = dv < 0 ? -dv - 1 : dv;
     const int drank = raw / a.NvS;
     const int loff = raw - drank * a.NvS;
-    const bool valid = lane < K && drank < a.R;  // never write outside the shards
-    const bool copy = valid && (dv >= 0 || (a.flags & MEP_DISPATCH_WRITE_DUPS));
-    if (valid && a.w) a.wslots[(size_t)drank * a.wslot_stride + loff] = a.w[(size_t)s * K + lane];
-    const uint64_t off = ((uint64_t)drank * (uint64_t)a.shard_stride_rows + (uint64_t)loff) * row_bytes;
-    const uint32_t off_lo = (uint32_t)off, off_hi = (uint32_t)(off >> 32);
-    uint64_t todo = __ballot(copy);
-    const char* src = (const char*)a.hidden + (size_t)s * row_bytes;
-    char* out = (char*)a.shards;
+    if (drank >= a.R) return;  // never write outside the shards
+    if (a.w && lane == 0) a.wslots[(size_t)drank * a.wslot_stride + loff] = a.w[gw];
+    if (dv < 0 && !(a.flags & MEP_DISPATCH_WRITE_DUPS)) return;
+    const char* src = (const char*)a.hidden + (size_t)s * row_bytes + (size_t)lane * 16;
+    char* row = (char*)a.shards +
+                ((uint64_t)drank * (uint64_t)a.shard_stride_rows + (uint64_t)loff) * row_bytes +
+                (size_t)lane * 16;
     if (NV > 0) {
       mep_u4 v[NV > 0 ? NV : 1];
 #pragma unroll
-      for (int i = 0; i < NV; ++i) v[i] = mep_ld16(src + ((size_t)i * 64 + lane) * 16);
-      while (todo) {
-        const int k = __ffsll((unsigned long long)todo) - 1;
-        todo &= todo - 1;
-        const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(off_hi, k) << 32) |
-                           (uint32_t)__builtin_amdgcn_readlane(off_lo, k);
-        char* row = out + o;
+      for (int i = 0; i < NV; ++i) v[i] = mep_ld16(src + (size_t)i * 1024);
 #pragma unroll
-        for (int i = 0; i < NV; ++i) mep_st16_stream(row + ((size_t)i * 64 + lane) * 16, v[i]);
-      }
+      for (int i = 0; i < NV; ++i) mep_st16_stream(row + (size_t)i * 1024, v[i]);
     } else {
       const int nvec = H / 8;
       for (int c0 = 0; c0 < nvec; c0 += 4 * 64) {
         mep_u4 v[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int c = c0 + i * 64 + lane;
-          if (c < nvec) v[i] = mep_ld16(src + (size_t)c * 16);
-        }
-        uint64_t t = todo;
-        while (t) {
-          const int k = __ffsll((unsigned long long)t) - 1;
-          t &= t - 1;
-          const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(off_hi, k) << 32) |
-                             (uint32_t)__builtin_amdgcn_readlane(off_lo, k);
-          char* row = out + o;
+        for (int i = 0; i < 4; ++i)
+          if (c0 + i * 64 + lane < nvec) v[i] = mep_ld16(src + (size_t)(c0 + i * 64) * 16);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int c = c0 + i * 64 + lane;
-            if (c < nvec) mep_st16_stream(row + (size_t)c * 16, v[i]);
-          }
-        }
+        for (int i = 0; i < 4; ++i)
+          if (c0 + i * 64 + lane < nvec) mep_st16_stream(row + (size_t)(c0 + i * 64) * 16, v[i]);
       }
     }
     return;
@@ -315,7 +296,7 @@ extern "C" int mep_dispatch(const void* hidden_SH, const float* w_SK, const int3
   a.shard_stride_rows = shard_stride_rows; a.wslot_stride = wslot_stride;
   a.rank = rank; a.S = S; a.H = H; a.K = K; a.R = R; a.NvS = NvS; a.flags = flags;
   a.groups = zf ? 2 * epn : 0;
-  a.tok_blocks = (S + kWavesPerBlock - 1) / kWavesPerBlock;
+  a.tok_blocks = (int)(((int64_t)S * K + kWavesPerBlock - 1) / kWavesPerBlock);
   int zpg = (token_padding - 1 + kWavesPerBlock - 1) / kWavesPerBlock;
   if (zpg > 32) zpg = 32;
   if (zpg < 1) zpg = 1;
