@@ -1,0 +1,77 @@
+"""End-to-end MoE layer on the emulated group: dispatch -> grouped FFN over
+(local experts + prefetch slots) -> combine, forward and backward through
+autograd, against a dense PyTorch MoE that never permutes anything.
+
+The communication ops are exact copies / ordered sums; what differs from the
+dense fp32 reference is bf16 rounding of rows and GEMM inputs, so values are
+compared at bf16-level tolerance (stated at the asserts)."""
+
+import pytest
+import torch
+
+from moonep_amd import moe, routing
+
+pytestmark = pytest.mark.gpu
+
+
+def _dense_reference(x, w, topk, master, epn):
+    """y[r,s] = sum_k w[r,s,k] * FFN_{topk[r,s,k]}(x[r,s]); bf16-rounded inputs, fp32 math."""
+    gate, up, down = (m.to(torch.bfloat16).float() for m in master)
+    R, S, K = topk.shape
+    xb = x.to(torch.bfloat16).float()
+    y = torch.zeros_like(xb)
+    for k in range(K):
+        e = topk[:, :, k].long()
+        g, u, d = gate[e // epn, e % epn], up[e // epn, e % epn], down[e // epn, e % epn]  # [R,S,H,Hp]
+        h = torch.nn.functional.silu(torch.einsum("rsh,rshp->rsp", xb, g)) * torch.einsum("rsh,rshp->rsp", xb, u)
+        y = y + w[:, :, k, None] * torch.einsum("rsp,rshp->rsh", h, d)
+    return y
+
+
+@pytest.mark.parametrize("sigma", [0.0, 2.0])
+def test_moe_layer_forward_backward_matches_dense(cuda, sigma):
+    R, epn, S, K, H, Hp, tp = 4, 2, 24, 3, 128, 128, 8
+    E = R * epn
+    topk = torch.stack([routing.popularity_biased(S, K, E, R, r, sigma, seed=5) for r in range(R)])
+    tpe = routing.tokens_per_expert(topk, E)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(R, S, H, generator=g).to(cuda).requires_grad_()
+    w = torch.softmax(torch.randn(R, S, K, generator=g), -1).to(cuda).requires_grad_()
+    master = [(torch.randn(R, epn, H, Hp, generator=g) * 0.08).to(cuda).requires_grad_() for _ in range(3)]
+    gout = torch.randn(R, S, H, generator=g).to(cuda)
+    topk_d, tpe_d = topk.to(cuda), tpe.to(cuda)
+
+    group = moe.EmulatedGroup(S, H, K, E, R, token_padding=tp)
+    rows, slots, cu, plans = moe.group_dispatch(group, x.to(torch.bfloat16), w, topk_d, tpe_d)
+    etc = plans[0].experts_to_copy
+    if sigma > 0:
+        assert bool((etc >= 0).any()), "the skewed routing must exercise prefetch slots"
+    views = [moe.group_compute_views(group, etc, m) for m in master]
+    y = torch.stack([moe.grouped_ffn(rows[r], slots[r], cu[r], views[0][r], views[1][r], views[2][r])
+                     for r in range(R)])
+    out = moe.group_combine(group, plans, y)
+    (out.float() * gout).sum().backward()
+    got = dict(out=out.float().detach(), x=x.grad.clone(), w=w.grad.clone(),
+               **{f"m{i}": m.grad.clone() for i, m in enumerate(master)})
+
+    for t in (x, w, *master):
+        t.grad = None
+    ref = _dense_reference(x, w, topk_d, master, epn)
+    (ref * gout).sum().backward()
+    want = dict(out=ref.detach(), x=x.grad, w=w.grad, **{f"m{i}": m.grad for i, m in enumerate(master)})
+
+    for name in want:
+        a, b = got[name], want[name]
+        scale = float(b.abs().max())
+        err = float((a - b).abs().max())
+        # bf16 has 8 significand bits: rows, GEMM inputs and the K-sum are each rounded
+        # once or twice on the way, so 3 % of the tensor's largest magnitude bounds it
+        assert err <= 0.03 * scale + 1e-6, (name, err, scale)
+        # and the direction agrees closely
+        cos = float(torch.nn.functional.cosine_similarity(a.flatten(), b.flatten(), dim=0))
+        assert cos > 0.999, (name, cos)
+    # experts never hosted remotely get grads only from their home rank; every
+    # master weight that received tokens has a non-zero grad
+    used = tpe.sum(0).reshape(R, epn) > 0
+    assert bool(((got["m0"].abs().amax(dim=(2, 3)) > 0).cpu() == used).all())
+    group.destroy()
