@@ -199,7 +199,26 @@ def cpu_baseline(ch, budget_s=20.0):
     ch.plan_fn(); ch.dispatch_fn(0); ch.combine_fn(0)   # the GPU's answer for the same token set
     torch.cuda.synchronize()
     got = ch.out[0].cpu().view(torch.int16).numpy().view(np.uint16)
+    # the same two data movements as torch-CPU index ops on every host core the
+    # process may use (the comparison the reference's own harness would make)
+    tdst = torch.from_numpy(dst.astype(np.int64))
+    rows = torch.where(tdst < 0, -tdst - 1, tdst)
+    th = ch.hidden[0].cpu()
+    tsh = torch.from_numpy(shards.view(np.int16)).view(torch.bfloat16).view(R * NvS, H)
+    tok = torch.arange(S).repeat_interleave(K)
+    tt = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        tsh.index_copy_(0, rows, th[tok])
+        t1 = time.perf_counter()
+        tout = tsh.index_select(0, rows).float().view(S, K, H).sum(1).to(torch.bfloat16)
+        t2 = time.perf_counter()
+        tt.append((t1 - t0, t2 - t1))
+    td, tc = min(tt, key=lambda t: sum(t))
     return {
+        "torch_cpu_threads": torch.get_num_threads(),
+        "torch_cpu_dispatch_GBps": ch.bytes_one_way() / td / 1e9,
+        "torch_cpu_combine_GBps": ch.bytes_one_way() / tc / 1e9,
         "value": 2 * ch.bytes_one_way() / total / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": f"full workload (S={S} tokens of one rank), best of {len(times) - 1} passes after 1 warm-up",
         "plan_us": p * 1e6, "dispatch_GBps": ch.bytes_one_way() / d / 1e9,

@@ -282,3 +282,28 @@ def test_chain_replays_from_a_hip_graph(cuda):
         for a, g in zip(want, got):
             assert torch.equal(a, g), seed
     b.destroy()
+
+
+def test_single_rank_group(cuda):
+    """R = 1: one rank is its own group; the [E]-shaped count vector of the
+    reference signature is accepted as is."""
+    S1, H1, K1, E1 = 20, 64, 2, 4
+    topk = routing.popularity_biased(S1, K1, E1, 1, 0, 1.0, seed=2)
+    tpe = routing.tokens_per_expert(topk, E1)
+    g = torch.Generator().manual_seed(2)
+    hid = torch.randn(S1, H1, generator=g).to(torch.bfloat16)
+    b = Buffer(S1, H1, K1, E1, 1, token_padding=4)
+    assert b._require_ctx()["rank"] == 0
+    h, w, cu, plan = b.dispatch(hid.to(cuda), None, topk.to(cuda), tpe.to(cuda))
+    out, _, _ = b.combine(plan=plan, hidden_nvsh=h)
+    torch.cuda.synchronize()
+    rp = po.plan(topk.numpy(), tpe.numpy().reshape(1, E1), 0, 4)
+    assert np.array_equal(plan.dst.cpu().numpy(), rp.dst)
+    assert (plan.experts_to_copy.cpu() == -1).all()
+    NvS = b._require_ctx()["NvS"]
+    sh = torch.zeros(1, NvS, H1, dtype=torch.bfloat16)
+    oo.dispatch(hid, None, torch.from_numpy(rp.dst), torch.from_numpy(rp.zero_fill_ranges), sh, None, 0, K1,
+                include_dups=True)
+    want, _ = oo.combine(sh, None, torch.from_numpy(rp.dst), K1, mode="two_level")
+    assert torch.equal(out.cpu().view(torch.int16), want.view(torch.int16))
+    b.destroy()

@@ -74,14 +74,18 @@ PLANS = {"ring": plan_ring, "fan_in": plan_fan_in, "empty": plan_empty,
          "asymmetric": plan_asymmetric, "random": plan_random}
 
 
-def strided_pool(R, per_rank_shape, dtype, pad_elems, fill, dev):
+def strided_pool(R, per_rank_shape, dtype, pad_elems, fill, dev, lead_elems=0):
     """[R, *per_rank_shape] view with `pad_elems` elements of padding between
-    ranks, everything (padding included) pre-filled with `fill`."""
+    ranks and `lead_elems` before the first, everything (padding included)
+    pre-filled with `fill`."""
     numel = 1
     for s in per_rank_shape:
         numel *= s
     stride = numel + pad_elems
-    backing = torch.full((R * stride,), fill, dtype=dtype, device=dev)
+    backing = torch.full((lead_elems + R * stride,), fill, dtype=dtype, device=dev)
+    if lead_elems:
+        whole = backing
+        backing = backing[lead_elems:]
     strides = [stride]
     acc = numel
     for s in per_rank_shape:
@@ -102,6 +106,7 @@ PREFETCH_CASES = [
     ("epn1", 2, 1, 128, 128, torch.bfloat16, "ring", 0, 0),
     ("uint8_packed", 4, 8, 256, 128, torch.uint8, "random", 3, 16),
     ("int8", 4, 3, 128, 384, torch.int8, "asymmetric", 0, 16),
+    ("offset_128B_pool", 4, 3, 384, 640, torch.bfloat16, "ring", 0, 64),
 ]
 
 
@@ -124,8 +129,9 @@ def test_prefetch_matches_oracle(cuda, case):
     locals_ = [[_fill((epn, *shp), dtype, g) for shp in shapes] for _ in range(R)]
     ref_pools, dev_pools, dev_backing = [], [], []
     for t, shp in enumerate(shapes):
-        _, rp = strided_pool(R, (epn, *shp), dtype, pad * (t + 1), sent, "cpu")
-        bk, dp = strided_pool(R, (epn, *shp), dtype, pad * (t + 1), sent, cuda)
+        lead = 64 * (t + 1) if name.startswith("offset") else 0   # 128-byte steps into the allocation
+        _, rp = strided_pool(R, (epn, *shp), dtype, pad * (t + 1), sent, "cpu", lead)
+        bk, dp = strided_pool(R, (epn, *shp), dtype, pad * (t + 1), sent, cuda, lead)
         ref_pools.append(rp)
         dev_pools.append(dp)
         dev_backing.append(bk)
