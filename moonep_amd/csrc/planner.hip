@@ -82,11 +82,13 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
     for (int r0 = 0; r0 < R; r0 += 8) {  // eight independent loads in flight
       int v[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = r0 + j < R ? a.tpe[(r0 + j) * E + e] : 0;
+      for (int j = 0; j < 8; ++j)  // clamped row: no branch between the loads
+        v[j] = a.tpe[(r0 + j < R ? r0 + j : R - 1) * E + e];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        if (r0 + j < rank) p += v[j];
-        c += v[j];
+        const int x = r0 + j < R ? v[j] : 0;
+        p += r0 + j < rank ? x : 0;
+        c += x;
       }
     }
     s_cnt[e] = c; s_prev[e] = p; s_rem[e] = c;
@@ -99,7 +101,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   // ---- receivers and quotas (wave 0) | histogram of earlier entries -------
   // Each receiver is filled exactly once (to capacity), so z[h][u] of the
   // reference (tests/planning_reference.py:85-96) is stored per receiver.
-  // The upper half of the waves meanwhile counts, per expert, this rank's
+  // The upper three quarters of the waves meanwhile count, per expert, this rank's
   // entries that precede the workgroup's slice: that needs nothing from the
   // plan and hides behind the serial greedy loops.
   const int* topk = a.topk + (size_t)blockIdx.y * N;
@@ -139,9 +141,9 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       if (lane == (u & 63)) { if (u < 64) b0 = 0; else b1 = 0; }
       if (lane == 0) { s_from[u] = h; s_quota[u] = move; }
     }
-  } else if (wave >= NW / 2) {
-    constexpr int HT = NT - (NW / 2) * 64;  // threads counting
-    const int ht = tid - (NW / 2) * 64;
+  } else if (wave >= NW / 4) {
+    constexpr int HT = NT - (NW / 4) * 64;  // threads counting
+    const int ht = tid - (NW / 4) * 64;
     int done = 0;
     if ((((uintptr_t)topk) & 15) == 0) {  // 16-byte loads, four in flight
       const int nv = e0 >> 2;
@@ -230,6 +232,8 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   __syncthreads();
 
   // ---- layout of every destination: one wave per destination -------------
+  const bool tp_pow2 = (tp & (tp - 1)) == 0;
+  const int epn_shift = (epn & (epn - 1)) == 0 ? 31 - __clz(epn) : -1;
   for (int d = wave; d < R; d += NW) {
     const int lo = d * epn, hi = lo + epn;
     int nremote = 0;
@@ -240,7 +244,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       if (sel) {
         const int slot = nremote + __popcll(m & mep_lanes_lt());
         if (slot < epn) s_etc[lo + slot] = e;
-        atomicAdd(&s_stat1[e / epn], 1);
+        atomicAdd(&s_stat1[epn_shift >= 0 ? e >> epn_shift : e / epn], 1);
       }
       nremote += __popcll(m);
     }
@@ -257,7 +261,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       if (g < epn) eid = lo + g;
       else if (g < 2 * epn) eid = s_etc[lo + g - epn];
       if (eid >= 0) cnt = alloc[eid * R + d];
-      const int padded = cnt > 0 ? ((cnt + tp - 1) / tp) * tp : 0;
+      const int padded = tp_pow2 ? (cnt + tp - 1) & ~(tp - 1) : ((cnt + tp - 1) / tp) * tp;
       const int incl = mep_wave_incl_scan(padded);
       const int start = running + incl - padded;
       if (cnt > 0) base[eid * R + d] = d * NvS + start;
@@ -315,10 +319,25 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
     // entries of expert e are numbered over (source rank, flat index) and cut
     // into the destinations' allocations in rank order
     int g = s_prev[e] + s_hist[e] + before + pos;
-    for (; dest < R - 1; ++dest) {
-      const int c = alloc[e * R + dest];
-      if (g < c) break;
-      g -= c;
+    if ((R & 3) == 0) {
+      const int4* row = (const int4*)(alloc + e * R);  // 16-byte aligned: tables start aligned, R % 4 == 0
+      bool found = false;
+      for (int d4 = 0; d4 < R && !found; d4 += 4) {
+        const int4 c4 = row[d4 >> 2];
+        const int cs[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (!found) {
+            if (g < cs[j] || d4 + j == R - 1) { dest = d4 + j; found = true; }
+            else g -= cs[j];
+          }
+      }
+    } else {
+      for (; dest < R - 1; ++dest) {
+        const int c = alloc[e * R + dest];
+        if (g < c) break;
+        g -= c;
+      }
     }
     dv = base[e * R + dest] + g;
   }
@@ -396,6 +415,7 @@ extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, in
   if (!c.lds_tables) {
     const size_t need = (size_t)c.groups * nranks * 2 * (size_t)E * R * sizeof(int);
     MEP_REQUIRE(scratch && scratch_bytes >= need, MEP_ERR_SCRATCH);
+    MEP_REQUIRE((uintptr_t)scratch % 16 == 0, MEP_ERR_ALIGNMENT);
   }
   PlanArgs a;
   a.tpe = tpe_RE; a.topk = topk_nSK; a.dst = dst; a.cu_seqlens = cu_seqlens;
