@@ -48,15 +48,24 @@ def parse():
 
 
 def time_launches(fn, iters, warmup=2):
-    """Average duration in microseconds of `fn`'s work on the current stream."""
+    """Average duration in microseconds of one `fn()` (a kernel launch on the current
+    stream): `iters` launches are captured into one HIP graph, so that host-side
+    launch cost (larger than a 10 us kernel when it comes from Python) stays out of
+    the figure; HIP events bracket the replay on the launching stream."""
     import torch
 
     for _ in range(warmup):
         fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(iters):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     a.record()
-    for _ in range(iters):
-        fn()
+    graph.replay()
     b.record()
     b.synchronize()
     return a.elapsed_time(b) * 1e3 / iters

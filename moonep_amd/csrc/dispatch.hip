@@ -19,7 +19,7 @@ struct DispatchArgs {
   uint16_t* shards;
   float* wslots;
   int64_t shard_stride_rows, wslot_stride;
-  int rank, S, H, K, R, NvS, groups, tok_blocks, zblocks_per_group;
+  int rank, S, H, K, R, NvS, groups, tok_blocks, zblocks, zblocks_per_group;
   unsigned flags;
 };
 
@@ -34,8 +34,10 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
   const int wave = threadIdx.x >> 6;
   const int H = a.H;
   const size_t row_bytes = (size_t)H * 2;
-  if ((int)blockIdx.x < a.tok_blocks) {
-    const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;  // flat (token, k) index
+  // the (few, short) zero-fill workgroups come first in the grid so that they
+  // overlap with the copies instead of forming a tail
+  if ((int)blockIdx.x >= a.zblocks) {
+    const int64_t gw = (int64_t)(blockIdx.x - a.zblocks) * kWavesPerBlock + wave;  // flat (token, k) index
     if (gw >= (int64_t)a.S * a.K) return;
     const int s = (int)(gw / a.K);
     const int dv = a.dst[gw];
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
     return;
   }
   // ---- zero-fill of this rank's padding rows (and their weight slots) -----
-  const int zb = blockIdx.x - a.tok_blocks;
+  const int zb = blockIdx.x;
   const int g = zb / a.zblocks_per_group;
   const int part = zb - g * a.zblocks_per_group;
   if (g >= a.groups) return;
@@ -303,6 +305,7 @@ extern "C" int mep_dispatch(const void* hidden_SH, const float* w_SK, const int3
   a.zblocks_per_group = zpg;
   const int zblocks = (zf && token_padding > 1) ? a.groups * zpg : 0;
   if (zblocks == 0) a.groups = 0;
+  a.zblocks = zblocks;
   dim3 grid(a.tok_blocks + zblocks);
   hipStream_t st = (hipStream_t)stream;
   const int nvec = H / 8;
