@@ -359,11 +359,13 @@ size_t plan_lds_bytes(int nt, int E, int R, bool lds_tables) {
   return ints * sizeof(int);
 }
 
-constexpr size_t kLdsDefaultLimit = 64 * 1024;
+constexpr size_t kLdsDefaultLimit = 64 * 1024;   // available to any kernel without opting in
+constexpr size_t kLdsOptInLimit = 160 * 1024;    // gfx950: what one workgroup can address
 
 struct PlanConfig {
   int nt;
   bool lds_tables;
+  bool opt_in;  // needs more dynamic LDS than the default limit
   size_t lds_bytes;
   int tok_per_wg;
   int groups;
@@ -371,12 +373,15 @@ struct PlanConfig {
 
 // 0 on success
 int plan_config(int S, int K, int E, int R, PlanConfig* c) {
+  c->opt_in = false;
   if (plan_lds_bytes(1024, E, R, true) <= kLdsDefaultLimit) {
     c->nt = 1024; c->lds_tables = true;
   } else if (plan_lds_bytes(256, E, R, true) <= kLdsDefaultLimit) {
     c->nt = 256; c->lds_tables = true;
   } else if (plan_lds_bytes(256, E, R, false) <= kLdsDefaultLimit) {
     c->nt = 256; c->lds_tables = false;
+  } else if (plan_lds_bytes(256, E, R, false) <= kLdsOptInLimit) {
+    c->nt = 256; c->lds_tables = false; c->opt_in = true;
   } else {
     return MEP_ERR_UNSUPPORTED;
   }
@@ -430,6 +435,12 @@ extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, in
   } else if (c.lds_tables) {
     hipLaunchKernelGGL((plan_kernel<256, true>), grid, dim3(256), c.lds_bytes, st, a);
   } else {
+    if (c.opt_in) {
+      hipError_t e = hipFuncSetAttribute((const void*)plan_kernel<256, false>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)kLdsOptInLimit);
+      if (e != hipSuccess) return (int)e;
+    }
     hipLaunchKernelGGL((plan_kernel<256, false>), grid, dim3(256), c.lds_bytes, st, a);
   }
   return mep_launch_status();

@@ -218,7 +218,8 @@ def test_combine_exact_cases(cuda):
     buf.destroy()
 
 
-@pytest.mark.parametrize("S,H,K,E,mv", [(4096, 7168, 8, 256, 1.0), (8192, 4096, 8, 128, 2.0)])
+@pytest.mark.parametrize("S,H,K,E,mv", [(4096, 7168, 8, 256, 1.0), (8192, 4096, 8, 128, 2.0),
+                                         (8192, 7168, 16, 256, 1.0)])  # last: 16 GB of shards, large strides
 def test_headline_shape_round_trip(cuda, S, H, K, E, mv):
     """Full-size single-rank share through the public API: properties that do
     not need an oracle pass over 4.7 GB."""

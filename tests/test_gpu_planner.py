@@ -98,6 +98,7 @@ def test_planner_matches_oracle_at_headline_shapes(cuda, S, H, K, E, R, mv):
     (128, 1, 64, 2, 8, 1.0),      # the encoding's rank limit
     (12, 70, 96, 5, 32, 1.0),     # more than 64 experts per rank
     (8, 8, 262144, 8, 128, 1.0),  # counts too large for packed (value, index) keys
+    (8, 512, 512, 4, 16, 1.0),    # E = 4096: per-expert arrays beyond 64 KB of LDS
 ])
 def test_planner_wide_groups_match_oracle(cuda, R, epn, S, K, tp, sigma):
     """Shapes outside the golden table (R > 8, large counts): the CPU oracle,

@@ -83,9 +83,7 @@ def strided_pool(R, per_rank_shape, dtype, pad_elems, fill, dev, lead_elems=0):
         numel *= s
     stride = numel + pad_elems
     backing = torch.full((lead_elems + R * stride,), fill, dtype=dtype, device=dev)
-    if lead_elems:
-        whole = backing
-        backing = backing[lead_elems:]
+    backing = backing[lead_elems:]
     strides = [stride]
     acc = numel
     for s in per_rank_shape:
@@ -167,8 +165,6 @@ def test_prefetch_with_scales_and_large_offsets(cuda):
         etc[d, 1] = ((d + 2) % R) * epn + 0
     g = torch.Generator().manual_seed(5)
     scale_shape = (64, 64)  # fp32: 16 KiB per expert = one re-tile unit
-    for rank in range(R):
-        pass
     locals_w = [[_fill((epn, H, Hp), torch.uint8, g) for _ in range(3)] for _ in range(R)]
     locals_s = [[torch.randn((epn, *scale_shape), generator=g) for _ in range(3)] for _ in range(R)]
     assert retile_for_prefetch(locals_s[0][0]).shape == (epn, 128, 128)
