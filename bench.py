@@ -111,7 +111,12 @@ class Chain:
         def combine_fn(i=0):
             launch_combine(ctx, self.out[i], self.plan.dst, self.out_w, mode="two_level")
 
+        def combine_weighted_fn(i=0):
+            # extension: sum_k w*row (the reference combine is unweighted); timed beside it
+            launch_combine(ctx, self.out[i], self.plan.dst, None, mode="weighted")
+
         self.plan_fn, self.dispatch_fn, self.combine_fn = plan_fn, dispatch_fn, combine_fn
+        self.combine_weighted_fn = combine_weighted_fn
         # eager once (also validates), then capture one graph per buffer set
         plan_fn(); dispatch_fn(); combine_fn()
         torch.cuda.synchronize()
@@ -167,13 +172,19 @@ def measure_chain(ch, steps, warmup):
     # the same token buffer every launch: rows stay in the last-level cache, as they
     # do when dispatch follows the kernel that produced them
     per["dispatch_us_warm_input"] = time_launches(lambda: ch.dispatch_fn(0), n)
+
+    def cw():
+        k[0] += 1
+        ch.combine_weighted_fn(k[0] % len(ch.out))
+
+    per["combine_weighted_us"] = time_launches(cw, n)
     by = ch.bytes_one_way()
     per["dispatch_GBps"] = by / per["dispatch_us"] / 1e3
     per["combine_GBps"] = by / per["combine_us"] / 1e3
     return wall_ms, ev_ms, per
 
 
-def cpu_baseline(ch, budget_s=20.0):
+def cpu_baseline(ch, budget_s=10.0):
     """Scalar C port of plan + dispatch + combine on the same inputs, host cores."""
     import numpy as np
     import torch
@@ -200,7 +211,7 @@ def cpu_baseline(ch, budget_s=20.0):
         out, out_w = co.combine(shards, wslots, dst, S, K, NvS, 2)
         t3 = time.perf_counter()
         times.append((t1 - t0, t2 - t1, t3 - t2))
-        if len(times) >= 2 and time.perf_counter() - t_all > budget_s or len(times) >= 8:
+        if len(times) >= 2 and time.perf_counter() - t_all > budget_s or len(times) >= 64:
             break
     # first pass pays the page faults of the fresh shards: report the best later pass
     p, d, c = min(times[1:], key=lambda t: sum(t))
@@ -229,7 +240,8 @@ def cpu_baseline(ch, budget_s=20.0):
         "torch_cpu_dispatch_GBps": ch.bytes_one_way() / td / 1e9,
         "torch_cpu_combine_GBps": ch.bytes_one_way() / tc / 1e9,
         "value": 2 * ch.bytes_one_way() / total / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-        "sample": f"full workload (S={S} tokens of one rank), best of {len(times) - 1} passes after 1 warm-up",
+        "sample": f"full workload (S={S} tokens of one rank), best of {len(times) - 1} passes after 1 warm-up "
+                  f"({time.perf_counter() - t_all:.0f} s of CPU work)",
         "plan_us": p * 1e6, "dispatch_GBps": ch.bytes_one_way() / d / 1e9,
         "combine_GBps": ch.bytes_one_way() / c / 1e9, "host_cpus": os.cpu_count(),
         "matches_gpu_output": bool(np.array_equal(out, got)),
@@ -324,6 +336,7 @@ def main():
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "graph_ms_per_step_events": ev_ms,
         "plan_us": per["plan_us"], "dispatch_us": per["dispatch_us"], "combine_us": per["combine_us"],
+        "combine_weighted_us": per["combine_weighted_us"],
         "dispatch_GBps": per["dispatch_GBps"], "combine_GBps": per["combine_GBps"],
         "dispatch_us_warm_input": per["dispatch_us_warm_input"],
         "dispatch_pct_hbm_peak": 100.0 * per["dispatch_GBps"] / HBM_PEAK_GBPS,

@@ -47,6 +47,11 @@ extern "C" {
 #define MEP_COMBINE_ALL 1       /* sum all K entries, one rounding                         */
 #define MEP_COMBINE_TWO_LEVEL 2 /* per-destination group sum -> bf16 -> sum (= reference
                                    prologue + combine, without modifying the shards)       */
+#define MEP_COMBINE_WEIGHTED 3  /* sum over all K entries of weight_slot * row; product and
+                                   sum rounded separately in fp32, one rounding to bf16.
+                                   Not a reference mode (its combine is unweighted): the
+                                   weighted top-k sum that callers otherwise apply on the
+                                   expert side                                              */
 
 int mep_version(void);
 const char* mep_strerror(int code);
@@ -67,8 +72,8 @@ size_t mep_plan_scratch_bytes(int S, int K, int E, int R, int nranks);
  *   cu_seqlens      [2*epn] out: padded end offset of each group on `rank`
  *   experts_to_copy [R,epn] out: remote experts every rank hosts (-1 = free)
  *   zero_fill       [2*epn,2] out: (first padding row, padding rows) per group
- *   remote_stats    [2]    out: (#experts I host for others' homes... i.e.
- *                          remote experts on me, #slots elsewhere holding mine)
+ *   remote_stats    [2]    out: (remote experts hosted on this rank,
+ *                          slots on other ranks that hold this rank's experts)
  * The src_info provenance scratch of the reference (planning.py:1036-1041)
  * is not produced; mep_build_dedup derives the duplicate groups from dst.
  */
@@ -130,7 +135,8 @@ int mep_combine_prologue(void* shard_NvS_H, const int32_t* dup_groups, const int
  * Top-k unpermute + K-sum + weight gather.  Replaces launch_combine
  * (reference moonep/combine.py:565-654; kernel :210-511).  Unweighted fp32
  * accumulation from +0.0 in ascending k, one round-to-nearest-even to bf16.
- *   out_SH [S,H] bf16; out_SK [S,K] fp32 or NULL (then wslots may be NULL)
+ *   out_SH [S,H] bf16; out_SK [S,K] fp32 or NULL (then wslots may be NULL unless the
+ *   mode is MEP_COMBINE_WEIGHTED)
  */
 int mep_combine(const void* shards, int64_t shard_stride_rows, const float* wslots,
                 int64_t wslot_stride, const int32_t* dst, void* out_SH, float* out_SK, int S,

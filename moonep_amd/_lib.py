@@ -20,6 +20,7 @@ _lib = None
 COMBINE_PRIMARIES = 0
 COMBINE_ALL = 1
 COMBINE_TWO_LEVEL = 2
+COMBINE_WEIGHTED = 3
 DISPATCH_WRITE_DUPS = 1
 DISPATCH_NO_ZERO_FILL = 2
 

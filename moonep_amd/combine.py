@@ -16,6 +16,7 @@ _MODES = {
     "primaries": _lib.COMBINE_PRIMARIES,
     "all": _lib.COMBINE_ALL,
     "two_level": _lib.COMBINE_TWO_LEVEL,
+    "weighted": _lib.COMBINE_WEIGHTED,
 }
 
 
@@ -46,7 +47,9 @@ def launch_combine(ctx: dict, output_sh, dst, output_sk=None, *, pdl_launch: boo
         every destination rank;
     mode "all": all K rows, one rounding;
     mode "two_level": all K rows, grouped and rounded exactly as prologue +
-        "primaries" would, without modifying the shards.
+        "primaries" would, without modifying the shards;
+    mode "weighted": not a reference mode -- all K rows, each multiplied by the
+        route weight in its slot (product and sum rounded separately in fp32).
     """
     assert output_sh.dtype == torch.bfloat16 and output_sh.is_contiguous(), \
         "output_sh must be contiguous bf16"
@@ -59,6 +62,7 @@ def launch_combine(ctx: dict, output_sh, dst, output_sk=None, *, pdl_launch: boo
         assert output_sk.dtype == torch.float32 and output_sk.is_contiguous(), \
             "output_sk must be contiguous fp32"
         assert output_sk.numel() == S * K
+    if output_sk is not None or mode == "weighted":
         wslots = ctx["meta_buf"].data_ptr() + 4 * int(ctx["WEIGHTS_OFF"])
     assert H % 8 == 0, "H must be a multiple of 8 (16-B row vectors)"
     rc = _lib.lib().mep_combine(

@@ -47,8 +47,9 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(CombineArgs a) {
   const int drank = raw / a.NvS;
   const int loff = raw - drank * a.NvS;
   const bool valid = lane < K && drank < a.R;
-  if (a.out_sk && part == 0 && lane < K)
-    a.out_sk[(size_t)s * K + lane] = valid ? a.wslots[(size_t)drank * a.wslot_stride + loff] : 0.0f;
+  float wk = 0.0f;  // route weight of entry `lane`, read from its slot
+  if (a.wslots && valid) wk = a.wslots[(size_t)drank * a.wslot_stride + loff];
+  if (a.out_sk && part == 0 && lane < K) a.out_sk[(size_t)s * K + lane] = wk;
   const uint64_t off = ((uint64_t)drank * (uint64_t)a.shard_stride_rows + (uint64_t)loff) * row_bytes;
   const uint32_t off_lo = (uint32_t)off, off_hi = (uint32_t)(off >> 32);
   const bool primary = valid && dv >= 0;
@@ -79,14 +80,31 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(CombineArgs a) {
   };
 
   if (!TWO) {
-    uint64_t t = a.mode == MEP_COMBINE_ALL ? valid_mask : prim_mask;
+    uint64_t t = a.mode == MEP_COMBINE_PRIMARIES ? prim_mask : valid_mask;
+    const bool weighted = a.mode == MEP_COMBINE_WEIGHTED;
     while (t) {
       const int k = __ffsll((unsigned long long)t) - 1;
       t &= t - 1;
       mep_u4 v[CH];
       load_row(row_of(k), v);
+      if (weighted) {
+        // acc += w * row with the product and the sum rounded separately
+        // (no fused multiply-add), in ascending k
+#pragma clang fp contract(off)
+        const float w = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(wk), k));
 #pragma unroll
-      for (int i = 0; i < CH; ++i) acc8(acc[i], v[i]);
+        for (int i = 0; i < CH; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float p0 = w * mep_bf16_lo(v[i][j]);
+            const float p1 = w * mep_bf16_hi(v[i][j]);
+            acc[i][2 * j] = acc[i][2 * j] + p0;
+            acc[i][2 * j + 1] = acc[i][2 * j + 1] + p1;
+          }
+      } else {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) acc8(acc[i], v[i]);
+      }
     }
   } else {
     // Per destination-rank group (its primary, then its duplicates in
@@ -162,10 +180,11 @@ extern "C" int mep_combine(const void* shards, int64_t shard_stride_rows, const 
   MEP_REQUIRE(shards && dst && out_SH, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(!out_SK || wslots, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(S > 0 && H > 0 && K > 0 && R > 0 && NvS > 0, MEP_ERR_INVALID_ARG);
-  MEP_REQUIRE(mode >= MEP_COMBINE_PRIMARIES && mode <= MEP_COMBINE_TWO_LEVEL, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(mode >= MEP_COMBINE_PRIMARIES && mode <= MEP_COMBINE_WEIGHTED, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(mode != MEP_COMBINE_WEIGHTED || wslots, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(K <= 32, MEP_ERR_UNSUPPORTED);
   MEP_REQUIRE(H % 8 == 0, MEP_ERR_UNSUPPORTED);
-  MEP_REQUIRE(shard_stride_rows >= NvS && (!out_SK || wslot_stride >= NvS), MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(shard_stride_rows >= NvS && (!wslots || wslot_stride >= NvS), MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(((uintptr_t)shards % 16 == 0) && ((uintptr_t)out_SH % 16 == 0), MEP_ERR_ALIGNMENT);
   CombineArgs a;
   a.shards = (const uint16_t*)shards; a.wslots = wslots; a.dst = dst;

@@ -86,6 +86,8 @@ def combine(shards, wslots, dst, K, mode="primaries"):
         of the group results in order of their primaries -- the bits the
         reference's prologue + combine pair produces, without touching the
         shards.
+    mode "weighted" (an extension, not in the reference): all K entries, each
+        row scaled by the fp32 route weight in its slot.
     Weight gather (reference moonep/combine.py:485-511): every entry reads its
     own slot.  Returns (out[S,H] bf16, weights[S,K] fp32 | None).
     """
@@ -119,6 +121,13 @@ def combine(shards, wslots, dst, K, mode="primaries"):
                 grp += torch.where(member[:, None], v, torch.zeros_like(v))
             grp = grp.to(torch.bfloat16).float()
             acc += torch.where(is_p[:, None], grp, torch.zeros_like(grp))
+        out = acc.to(torch.bfloat16)
+    elif mode == "weighted":
+        # not a reference mode: sum_k w[s,k] * row_k, product and sum each rounded to fp32
+        wk = wslots.view(-1)[drank * NvS + loff].view(S, K)
+        acc = torch.zeros(S, H, dtype=torch.float32)
+        for k in range(K):
+            acc += wk[:, k:k + 1] * flat[rows[:, k]].float()
         out = acc.to(torch.bfloat16)
     else:
         raise ValueError(mode)

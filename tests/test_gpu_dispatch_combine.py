@@ -158,6 +158,18 @@ def test_world_dispatch_combine_matches_oracle(cuda, case):
             assert torch.equal(out_w.cpu().view(torch.int32), want_w.view(torch.int32))
             # the gathered weights are the ones this rank scattered
             assert torch.equal(out_w.cpu().view(torch.int32), wts[r].view(torch.int32))
+    # weighted extension: bit-exact against the oracle that rounds product and sum separately
+    # (ordinary route weights: the traceable ones above are bit patterns, not magnitudes)
+    ws_w = torch.rand(R, NvS, generator=g) * 0.95 + 0.05
+    world.meta_buf.view(R, mcp)[:, :NvS] = ws_w.view(torch.int32).to(cuda)
+    for r in range(R):
+        dst_r = torch.from_numpy(plans[r].dst)
+        want, _ = oo.combine(expert_out, ws_w, dst_r, K, mode="weighted")
+        out = torch.empty(S, H, dtype=torch.bfloat16, device=cuda)
+        launch_combine(bufs[r]._require_ctx(), out, gplans[r].dst, None, mode="weighted")
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu().view(torch.int16), want.view(torch.int16)), ("weighted", r)
+    world.meta_buf.view(R, mcp)[:, :NvS] = ws_ref.view(torch.int32).to(cuda)
     # Tolerance of the reference's own test (tests/test_combine.py:202-211):
     # within 1 bf16 ulp (+0.5 slack) of the single-rounding fp32 K-sum, on
     # same-sign data (with cancellation the group rounding of the reference

@@ -97,6 +97,17 @@ def test_combine_closed_forms():
     for mode in ("all", "two_level"):
         out, _ = oo.combine(ints, None, dst, K, mode=mode)
         assert torch.equal(out, want)
+    # weighted mode: power-of-two weights and small integers keep every product and
+    # partial sum exact, so the result is the plain weighted sum; weight 1 reduces to "all"
+    w2 = (2.0 ** torch.randint(-3, 3, (R, NvS), generator=g).float())
+    wk = w2.view(-1)[drank * NvS + loff].view(S, K, 1)
+    want_w = (ints.view(-1, H)[drank * NvS + loff].float().view(S, K, H) * wk).sum(1)
+    out, _ = oo.combine(ints, w2, dst, K, mode="weighted")
+    assert torch.equal(out, want_w.to(torch.bfloat16))
+    rnd = torch.randn(R, NvS, H, generator=g).to(torch.bfloat16)
+    a, _ = oo.combine(rnd, torch.ones(R, NvS), dst, K, mode="weighted")
+    b, _ = oo.combine(rnd, None, dst, K, mode="all")
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     # dispatch then combine returns K * token (up to the rounding of the sum)
     hid = (torch.randn(S, H, generator=g)).to(torch.bfloat16)
     sh = torch.zeros(R, NvS, H, dtype=torch.bfloat16)
