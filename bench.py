@@ -235,10 +235,20 @@ def cpu_baseline(ch, budget_s=10.0):
         t2 = time.perf_counter()
         tt.append((t1 - t0, t2 - t1))
     td, tc = min(tt, key=lambda t: sum(t))
+    nthreads = torch.get_num_threads()
+    torch.set_num_threads(1)
+    t0 = time.perf_counter()
+    tsh.index_copy_(0, rows, th[tok])
+    t1 = time.perf_counter()
+    tsh.index_select(0, rows).float().view(S, K, H).sum(1).to(torch.bfloat16)
+    t2 = time.perf_counter()
+    torch.set_num_threads(nthreads)
     return {
-        "torch_cpu_threads": torch.get_num_threads(),
+        "torch_cpu_threads": nthreads,
         "torch_cpu_dispatch_GBps": ch.bytes_one_way() / td / 1e9,
         "torch_cpu_combine_GBps": ch.bytes_one_way() / tc / 1e9,
+        "torch_cpu_1thread_dispatch_GBps": ch.bytes_one_way() / (t1 - t0) / 1e9,
+        "torch_cpu_1thread_combine_GBps": ch.bytes_one_way() / (t2 - t1) / 1e9,
         "value": 2 * ch.bytes_one_way() / total / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": f"full workload (S={S} tokens of one rank), best of {len(times) - 1} passes after 1 warm-up "
                   f"({time.perf_counter() - t_all:.0f} s of CPU work)",
@@ -296,6 +306,28 @@ def bench_weights(seed, steps):
         by = (n_slots + 2 * active + own_slots) * per * 4   # slots read, grads read+written, clears
         res[name].update({"grad_reduce_us": us, "grad_reduce_bytes": by,
                           "grad_reduce_GBps": by / us / 1e3 if by else 0.0})
+    del grad, red
+    torch.cuda.empty_cache()
+    # host-core figures on a bounded sample: 4 slot copies (index_copy_) and 4 slot sums
+    # (add_ then zero_) of one projection, all torch threads
+    n = 4
+    lc = (torch.randn(n, H, Hp) * 0.02).to(torch.bfloat16)
+    pc = torch.empty(2 * n, H, Hp, dtype=torch.bfloat16)
+    idx = torch.arange(n) * 2 + 1
+    pc.index_copy_(0, idx, lc)
+    t0 = time.perf_counter()
+    pc.index_copy_(0, idx, lc)
+    t1 = time.perf_counter()
+    gc, rc = torch.zeros(n, H, Hp), torch.randn(n, H, Hp) * 1e-3
+    t2 = time.perf_counter()
+    for i in range(n):
+        gc[i].add_(rc[i])
+        rc[i].zero_()
+    t3 = time.perf_counter()
+    res["cpu_baseline"] = {
+        "torch_cpu_threads": torch.get_num_threads(), "sample": f"{n} slots of one projection",
+        "prefetch_GBps": 2 * n * per * 2 / (t1 - t0) / 1e9,
+        "grad_reduce_GBps": 4 * n * per * 4 / (t3 - t2) / 1e9}
     return res
 
 
