@@ -308,26 +308,31 @@ def bench_weights(seed, steps):
                           "grad_reduce_GBps": by / us / 1e3 if by else 0.0})
     del grad, red
     torch.cuda.empty_cache()
-    # host-core figures on a bounded sample: 4 slot copies (index_copy_) and 4 slot sums
-    # (add_ then zero_) of one projection, all torch threads
-    n = 4
+    # host-core figures on a bounded sample of one projection: 16 slot copies
+    # (index_copy_) and 8 slot sums (add_ then zero_), all torch threads; a 1 GiB
+    # fill between warm-up and timing pushes the sample out of the host caches
+    n, m = 16, 8
     lc = (torch.randn(n, H, Hp) * 0.02).to(torch.bfloat16)
     pc = torch.empty(2 * n, H, Hp, dtype=torch.bfloat16)
     idx = torch.arange(n) * 2 + 1
+    gc, rc = torch.zeros(m, H, Hp), torch.randn(m, H, Hp) * 1e-3
     pc.index_copy_(0, idx, lc)
+    flush = torch.empty(1 << 28, dtype=torch.float32)
+    flush.fill_(1.0)
     t0 = time.perf_counter()
     pc.index_copy_(0, idx, lc)
     t1 = time.perf_counter()
-    gc, rc = torch.zeros(n, H, Hp), torch.randn(n, H, Hp) * 1e-3
+    flush.fill_(2.0)
     t2 = time.perf_counter()
-    for i in range(n):
+    for i in range(m):
         gc[i].add_(rc[i])
         rc[i].zero_()
     t3 = time.perf_counter()
     res["cpu_baseline"] = {
-        "torch_cpu_threads": torch.get_num_threads(), "sample": f"{n} slots of one projection",
+        "torch_cpu_threads": torch.get_num_threads(),
+        "sample": f"{n} slot copies / {m} slot sums of one projection",
         "prefetch_GBps": 2 * n * per * 2 / (t1 - t0) / 1e9,
-        "grad_reduce_GBps": 4 * n * per * 4 / (t3 - t2) / 1e9}
+        "grad_reduce_GBps": 4 * m * per * 4 / (t3 - t2) / 1e9}
     return res
 
 

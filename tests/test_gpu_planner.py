@@ -124,3 +124,52 @@ def test_planner_wide_groups_match_oracle(cuda, R, epn, S, K, tp, sigma):
     assert np.array_equal(zfr.cpu().numpy(), gp.zero_fill)
     assert np.array_equal(stats.cpu().numpy(), gp.remote_stats)
     buf.destroy()
+
+
+def test_planner_random_small_shapes_match_oracle(cuda):
+    """Seeded sweep of small shapes with awkward routing: equal balances (ties in
+    every argmax/argmin), experts nobody routes to, one hot expert, repeated
+    experts inside a token, padding 1 and padding larger than any group."""
+    rng = np.random.default_rng(20240)
+    checked = 0
+    for it in range(120):
+        R = int(rng.choice([1, 2, 3, 4, 5, 8]))
+        epn = int(rng.integers(1, 6))
+        K = int(rng.integers(1, 5))
+        S = int(rng.integers(1, 49))
+        tp = int(rng.choice([1, 2, 4, 16, 64]))
+        E = R * epn
+        kind = it % 4
+        if kind == 0:      # uniform with replacement: duplicates inside a token
+            topk = rng.integers(0, E, (R, S, K))
+        elif kind == 1:    # every rank sends every token to the same few experts
+            hot = rng.integers(0, E, (max(1, min(E, 2)),))
+            topk = hot[rng.integers(0, hot.size, (R, S, K))]
+        elif kind == 2:    # identical routing on every rank: equal balances everywhere
+            one = rng.integers(0, E, (1, S, K))
+            topk = np.repeat(one, R, axis=0)
+        else:              # skewed popularity, distinct experts per token where possible
+            p = np.exp(rng.normal(0.0, 2.0, E))
+            p /= p.sum()
+            topk = np.stack([[rng.choice(E, K, replace=K > E, p=p) for _ in range(S)]
+                             for _ in range(R)])
+        topk = topk.astype(np.int32)
+        tpe = np.stack([np.bincount(topk[r].reshape(-1), minlength=E) for r in range(R)]).astype(np.int32)
+        try:
+            gp, plans, dst_all_ref = oracle_world_plan(topk, tpe, tp)
+        except AssertionError:
+            continue   # more remote experts than slots on some rank: the reference asserts too
+        buf = Buffer(S, 16, K, E, R, token_padding=tp, rank=0)
+        dst_all, cu, etc, zfr, stats = launch_planning_all_ranks(
+            buf._require_ctx(), torch.from_numpy(topk).to(cuda), torch.from_numpy(tpe).to(cuda))
+        torch.cuda.synchronize()
+        tag = f"iter {it}: R={R} epn={epn} S={S} K={K} tp={tp} kind={kind}"
+        assert np.array_equal(dst_all.cpu().numpy(), dst_all_ref), tag
+        assert np.array_equal(cu.cpu().numpy(), gp.cu_seqlens), tag
+        assert np.array_equal(etc.cpu().numpy(), gp.experts_to_copy), tag
+        assert np.array_equal(zfr.cpu().numpy(), gp.zero_fill), tag
+        assert np.array_equal(stats.cpu().numpy(), gp.remote_stats), tag
+        buf.destroy()
+        checked += 1
+    print(f"{checked} random shapes checked", flush=True)
+    assert checked >= 80
