@@ -57,6 +57,24 @@ CASES = [
 ]
 
 
+def _random_cases(n, seed=99):
+    """Seeded small shapes: row lengths that are odd multiples of 8 elements, K
+    up to 6, 1 to 8 ranks, paddings from 1 to 64."""
+    import random
+    rnd = random.Random(seed)
+    out = []
+    for i in range(n):
+        R = rnd.choice([1, 2, 3, 4, 8])
+        epn = rnd.randint(1, 5)
+        K = rnd.randint(1, min(6, R * epn))
+        out.append((f"rand{i}", rnd.randint(1, 40), 8 * rnd.randint(1, 160), K, epn, R,
+                    rnd.choice([1, 4, 16, 64]), ("biased", rnd.choice([0.0, 1.0, 3.0]))))
+    return out
+
+
+CASES += _random_cases(24)
+
+
 def _topk(case):
     name, S, H, K, epn, R, tp, (kind, arg) = case
     E = epn * R
