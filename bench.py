@@ -29,7 +29,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM-side bytes per launch (L2 fetches + writes) from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs, scaled by the factors a 512 MiB copy gives (2.000 and 1.000);
 # the summary is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"dispatch": 119.7e6 + 498.5e6, "combine": 471.3e6 + 58.9e6}
+MEASURED_TRAFFIC_BYTES = {"dispatch": 119.7e6 + 498.4e6, "combine": 472.0e6 + 58.9e6}
 
 
 def parse():
