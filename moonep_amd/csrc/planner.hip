@@ -12,6 +12,8 @@
 // (reference tests/planning_reference.py:25-311).
 #include "mep_common.h"
 
+#include <atomic>
+
 namespace {
 
 struct PlanArgs {
@@ -436,10 +438,18 @@ extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, in
     hipLaunchKernelGGL((plan_kernel<256, true>), grid, dim3(256), c.lds_bytes, st, a);
   } else {
     if (c.opt_in) {
-      hipError_t e = hipFuncSetAttribute((const void*)plan_kernel<256, false>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)kLdsOptInLimit);
+      // once per device: later launches (also under stream capture) find it set
+      static std::atomic<uint64_t> opted{0};
+      int dev = 0;
+      hipError_t e = hipGetDevice(&dev);
       if (e != hipSuccess) return (int)e;
+      const uint64_t bit = 1ull << (dev & 63);
+      if (!(opted.load(std::memory_order_acquire) & bit)) {
+        e = hipFuncSetAttribute((const void*)plan_kernel<256, false>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsOptInLimit);
+        if (e != hipSuccess) return (int)e;
+        opted.fetch_or(bit, std::memory_order_release);
+      }
     }
     hipLaunchKernelGGL((plan_kernel<256, false>), grid, dim3(256), c.lds_bytes, st, a);
   }
