@@ -71,12 +71,14 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(CombineArgs a) {
                        (uint32_t)__builtin_amdgcn_readlane(off_lo, k);
     return base + o;
   };
+  // chunks past the end of a ragged row re-read the row's first vector (their
+  // sums are never stored): loads stay unconditional
+  int voff[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) voff[i] = (EXACT || c0 + i * 64 < nvec) ? i * 1024 : -c0 * 16;
   auto load_row = [&](const char* row, mep_u4* v) {
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      v[i] = mep_u4{0u, 0u, 0u, 0u};
-      if (EXACT || c0 + i * 64 < nvec) v[i] = mep_ld16_stream(row + (size_t)i * 1024);
-    }
+    for (int i = 0; i < CH; ++i) v[i] = mep_ld16_stream(row + voff[i]);
   };
 
   if (!TWO) {
