@@ -89,9 +89,19 @@ size_t slot_table_bytes(int R, int epn) {
 // stream a little faster (6.3 vs 5.9 TB/s at 32768 vs 2048 for a dense slot
 // table) but each pays the table set-up, which dominates when only a few
 // experts are hosted remotely -- the common case; 4096 balances the two.
-int stream_blocks(int64_t work, int R, int epn) {
+// The number of active experts is only known on the device, so the grid is
+// sized from the tiles of ONE expert: with `tiles` (or an even fraction of
+// them) workgroups every workgroup moves the same number of tiles whatever
+// that number is; small tensors spread over up to `epn` experts' tiles.
+int stream_blocks(int64_t tiles, int R, int epn) {
   const int64_t cap = (int64_t)R * epn <= 1024 ? 4096 : 2048;
-  return (int)(work < cap ? (work > 0 ? work : 1) : cap);
+  if (tiles <= 0) return 1;
+  if (8 * tiles > cap) {
+    const int64_t per_block = (tiles + cap - 1) / cap;  // tiles of an expert per workgroup
+    return (int)((tiles + per_block - 1) / per_block);
+  }
+  const int64_t all = tiles * epn;
+  return (int)(all < cap ? all : cap / tiles * tiles);
 }
 
 struct PrefetchArgs {
@@ -287,7 +297,7 @@ extern "C" int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t ra
   ReduceArgs a{local_grad, reduce_pool, rank_stride_elems, elems_per_expert, experts_to_copy,
                rank, epn, R};
   const int64_t tiles = (elems_per_expert / 4 + kBlock * kVecPerThread - 1) /
-                        (kBlock * kVecPerThread) * epn;
+                        (kBlock * kVecPerThread);
   const int blocks = stream_blocks(tiles, R, epn);
   hipStream_t st = (hipStream_t)stream;
   // two launches: the clear must not overtake reads of a slot that holds one
