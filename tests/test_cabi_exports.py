@@ -56,3 +56,37 @@ def test_missing_library_is_a_loud_error(monkeypatch, tmp_path):
         assert "no CPU or eager fallback" in str(e)
     else:
         raise AssertionError("expected RuntimeError")
+
+
+def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
+    """Specific MEP_ERR_* codes; every check sits before the launch, so fake
+    (never dereferenced) device addresses are enough and no GPU is needed."""
+    lib = _lib.lib()
+    A = 0x10000          # 16-byte aligned stand-in for a device pointer
+    ok_plan = dict(S=4, K=2, E=8, R=2, tp=8, NvS=64)
+
+    def plan(**kw):
+        a = dict(ok_plan, scratch=None, sbytes=0)
+        a.update(kw)
+        return lib.mep_plan(A, A, 0, a["S"], a["K"], a["E"], a["R"], a["tp"], a["NvS"], A, A, A, A, A,
+                            a["scratch"], a["sbytes"], None)
+
+    assert plan(K=33) == -2                      # more than 32 routes per token
+    assert plan(R=3) == -1                       # E not divisible by R
+    assert plan(NvS=4) == -2                     # NvS below S*K
+    assert plan(R=2, NvS=1 << 30) == -2          # R*NvS does not fit the int32 encoding
+    assert plan(E=2050, S=256, K=1, NvS=1024) == -3        # planner tables need caller scratch
+    assert plan(E=2050, S=256, K=1, NvS=1024, scratch=A + 4, sbytes=1 << 30) == -4   # misaligned scratch
+    assert plan(E=1 << 16, R=2, S=256, K=1, NvS=1024, scratch=A, sbytes=1 << 40) == -2  # beyond the LDS limit
+    # dispatch / combine: misaligned rows, weights without slots, bad mode, ragged H
+    assert lib.mep_dispatch(A + 2, None, A, A, A, 64, None, 0, 0, 4, 64, 2, 2, 4, 64, 8, 0, None) == -4
+    assert lib.mep_dispatch(A, A, A, A, A, 64, None, 0, 0, 4, 64, 2, 2, 4, 64, 8, 0, None) == -1
+    assert lib.mep_dispatch(A, None, A, A, A, 64, None, 0, 5, 4, 64, 2, 2, 4, 64, 8, 0, None) == -1  # rank >= R
+    assert lib.mep_combine(A, 64, None, 0, A, A, None, 4, 64, 2, 2, 64, 7, None) == -1     # unknown mode
+    assert lib.mep_combine(A, 64, None, 0, A, A, None, 4, 64, 2, 2, 64, 3, None) == -1     # weighted without slots
+    assert lib.mep_combine(A, 64, None, 0, A, A, None, 4, 60, 2, 2, 64, 0, None) == -2     # H % 8 != 0
+    assert lib.mep_combine(A, 64, None, 0, A, A, None, 4, 64, 33, 2, 64, 0, None) == -2    # K > 32
+    assert lib.mep_combine(A, 32, None, 0, A, A, None, 4, 64, 2, 2, 64, 0, None) == -1     # stride < NvS
+    assert lib.mep_grad_reduce(A, A, 16 * 4, A, 0, 4, 2, 18, None) == -2                   # elems % 4 != 0
+    assert lib.mep_grad_reduce(A, A, 8, A, 0, 4, 2, 16, None) == -1                        # stride too small
+    assert lib.mep_grad_reduce(A + 4, A, 64, A, 0, 4, 2, 16, None) == -4
