@@ -295,3 +295,84 @@ def test_headline_shape_round_trip(cuda, S, H, K, E, mv):
     torch.cuda.synchronize()
     assert bool((out1 == float(K)).all())
     buf.destroy()
+
+
+def test_saved_plan_hidden_only_dispatch_reuses_dst_and_skips_weights(cuda):
+    """Mirror of reference tests/test_dispatch.py:351-416: a plan saved from an
+    earlier dispatch is reused for a hidden-only dispatch after another plan
+    has used the buffers.  The rows must follow the saved dst, the padding rows
+    must be zero, the weight slots must keep what the other dispatch left and
+    the saved duplicate structures must not change."""
+    from moonep_amd.planning import allocate_planning_outputs, launch_planning, \
+        launch_planning_all_ranks
+
+    S, K, epn, H, tp, R = 17, 3, 8, 64, 16, 4
+    E = R * epn
+    world = EmulatedWorld(S, H, K, E, R, tp)
+    bufs = [Buffer(S, H, K, E, R, token_padding=tp, rank=r, world=world) for r in range(R)]
+    NvS = world.NvS
+    mcp = world.layout["meta_chunk_padded"]
+
+    def plan_all(kind):
+        topk = torch.stack([routing.pattern(kind, S, K, E, R, r) for r in range(R)])
+        tpe = routing.tokens_per_expert(topk, E).to(cuda)
+        dst_all = launch_planning_all_ranks(bufs[0]._require_ctx(), topk.to(cuda), tpe)[0]
+        plans = []
+        for r in range(R):
+            plan, cu = allocate_planning_outputs(bufs[r]._require_ctx())
+            launch_planning(bufs[r]._require_ctx(), topk[r].reshape(-1).to(cuda), tpe, cu, plan)
+            plans.append(plan)
+        return plans, dst_all
+
+    hid_a = [traceable_hidden(S, H, r).to(cuda) for r in range(R)]
+    wts_a = [traceable_weights(S, K, r).to(cuda) for r in range(R)]
+    plans_a, dst_all_a = plan_all("all_remote")
+    for r in range(R):
+        launch_dispatch(bufs[r]._require_ctx(), hid_a[r], wts_a[r], plans_a[r], build_dedup_map=True,
+                        dst_all_ranks=dst_all_a)
+    for r in range(R):
+        launch_dispatch_epilogue(bufs[r]._require_ctx(), plans_a[r])
+    torch.cuda.synchronize()
+    saved = [(p.dup_groups.clone(), p.dup_loffs.clone(), p.dup_counts.clone()) for p in plans_a]
+    assert sum(int(c[2][1]) for c in saved) > 0, "the saved plans should hold duplicates"
+
+    g = torch.Generator().manual_seed(3)
+    plans_b, dst_all_b = plan_all("all_local")
+    for r in range(R):
+        hb = torch.randn(S, H, generator=g).to(torch.bfloat16).to(cuda)
+        wb = torch.rand(S, K, generator=g).to(cuda)
+        launch_dispatch(bufs[r]._require_ctx(), hb, wb, plans_b[r], build_dedup_map=True,
+                        dst_all_ranks=dst_all_b)
+    for r in range(R):
+        launch_dispatch_epilogue(bufs[r]._require_ctx(), plans_b[r])
+    torch.cuda.synchronize()
+    weights_after_b = world.meta_buf.view(R, mcp)[:, :NvS].clone()
+
+    for r in range(R):   # the reuse: no weights, no duplicate-map build
+        launch_dispatch(bufs[r]._require_ctx(), hid_a[r], None, plans_a[r], build_dedup_map=False)
+    for r in range(R):
+        launch_dispatch_epilogue(bufs[r]._require_ctx(), plans_a[r])
+    torch.cuda.synchronize()
+
+    shards = world.hidden_buf.view(R, NvS, H).cpu()
+    checked = 0
+    for r in range(R):
+        drank, loff, _ = oo.decode(plans_a[r].dst.cpu(), NvS)
+        rows = shards[drank, loff]                      # [S*K, H], duplicates included
+        want = hid_a[r].cpu().repeat_interleave(K, dim=0)
+        assert torch.equal(rows.view(torch.int16), want.view(torch.int16)), f"rank {r} rows"
+        checked += rows.shape[0]
+        padded = 0
+        for start, n in plans_a[r].zero_fill_ranges.cpu().tolist():
+            if n:
+                assert (shards[r, start:start + n] == 0).all()
+                padded += n
+        assert padded > 0
+    assert checked == R * S * K
+    assert torch.equal(world.meta_buf.view(R, mcp)[:, :NvS], weights_after_b), \
+        "weight slots changed during a hidden-only dispatch"
+    for p, (dg, dl, dc) in zip(plans_a, saved):
+        assert torch.equal(p.dup_groups, dg) and torch.equal(p.dup_loffs, dl) and \
+            torch.equal(p.dup_counts, dc), "saved duplicate structures changed during reuse"
+    for b in bufs:
+        b.destroy()
