@@ -278,6 +278,24 @@ def cpu_baseline(ch, budget_s=10.0):
     }
 
 
+def gpu_plan_all_ranks(S, K, E, R, tp, topk, tpe):
+    """All ranks' plans from the HIP planner: (cu_seqlens [R,2*epn] on the device,
+    experts_to_copy [R,epn] as numpy, NvS)."""
+    import torch
+
+    from moonep_amd import Buffer
+    from moonep_amd.planning import launch_planning_all_ranks
+
+    buf = Buffer(S, 16, K, E, R, token_padding=tp, rank=0)   # H plays no part in planning
+    ctx = buf._require_ctx()
+    dev = torch.device("cuda", 0)
+    _, cu, etc, _, _ = launch_planning_all_ranks(ctx, topk.to(dev), tpe.to(dev))
+    torch.cuda.synchronize()
+    out = cu.clone(), etc.cpu().numpy().astype("int64"), int(ctx["NvS"])
+    buf.destroy()
+    return out
+
+
 def bench_weights(seed, steps):
     """prefetch_weight (3 projections, one launch) and reduce_grad (one projection) at
     H=7168, H'=2048, epn=32, R=8 for two slot tables: the planner's own at maxvio~1
@@ -288,13 +306,12 @@ def bench_weights(seed, steps):
     from moonep_amd import routing
     from moonep_amd.grad_reduce import launch_grad_reduce
     from moonep_amd.prefetch import launch_prefetch
-    from oracle import planner_oracle as po
 
     S, K, E, R, H, Hp = 4096, 8, 256, 8, 7168, 2048
     epn = E // R
     dev = torch.device("cuda", 0)
     topk, _, tpe, mv, _ = routing.logit_routing(S, K, E, R, 1.0, seed, want_weights=False)
-    planned = po.plan_global(tpe.numpy(), S, K, 128).experts_to_copy
+    planned = gpu_plan_all_ranks(S, K, E, R, 128, topk, tpe)[1]
     ring = -np.ones((R, epn), dtype=np.int64)
     for d in range(R):
         for b in range(8):
@@ -354,6 +371,48 @@ def bench_weights(seed, steps):
         "prefetch_GBps": 2 * n * per * 2 / (t1 - t0) / 1e9,
         "grad_reduce_GBps": 4 * m * per * 4 / (t3 - t2) / 1e9}
     return res
+
+
+def bench_ffn(seed, steps):
+    """Expert-side consumer at the real shape: one rank's dispatched rows
+    (planner's own cu_seqlens at maxvio ~ 1, NvS = 40960 rows, H = 7168) through
+    the grouped SwiGLU gate/up GEMM (H' = 2048) and the grouped down GEMM, 64
+    groups.  FLOPs count the rows inside groups (padding rows included)."""
+    import torch
+
+    from moonep_amd import routing
+    from moonep_amd.ffn import launch_grouped_gemm_nt
+
+    S, K, E, R, H, Hp = 4096, 8, 256, 8, 7168, 2048
+    G = 2 * (E // R)
+    dev = torch.device("cuda", 0)
+    topk, _, tpe, mv, _ = routing.logit_routing(S, K, E, R, 1.0, seed, want_weights=False)
+    cu_all, _, NvS = gpu_plan_all_ranks(S, K, E, R, 128, topk, tpe)
+    cu = cu_all[0].contiguous()
+    used = int(cu[-1])
+    g = torch.Generator(device=dev).manual_seed(seed)
+    rows = torch.randn(NvS, H, device=dev, generator=g).to(torch.bfloat16)
+    gate = (torch.randn(G, Hp, H, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    up = (torch.randn(G, Hp, H, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    down = (torch.randn(G, H, Hp, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    slots = torch.rand(NvS, device=dev, generator=g)
+    hmid = torch.zeros(NvS, Hp, dtype=torch.bfloat16, device=dev)
+    out = torch.zeros(NvS, H, dtype=torch.bfloat16, device=dev)
+    t1 = time_launches(lambda: launch_grouped_gemm_nt(rows, gate, cu, hmid, up_weights=up), steps)
+    t2 = time_launches(lambda: launch_grouped_gemm_nt(hmid, down, cu, out, row_scale=slots), steps)
+    f1, f2 = 4.0 * used * H * Hp, 2.0 * used * H * Hp
+    # the library's dense GEMM of the same volume, for scale (one weight matrix, no groups)
+    c = torch.empty(used, Hp, dtype=torch.bfloat16, device=dev)
+    t3 = time_launches(lambda: torch.matmul(rows[:used], gate[0].t(), out=c), steps)
+    peak = 2500.0
+    return {
+        "rows_in_groups": used, "NvS": NvS, "groups": G, "maxvio": mv,
+        "swiglu_gate_up_us": t1, "swiglu_gate_up_TFLOPs": f1 / t1 / 1e6,
+        "down_us": t2, "down_TFLOPs": f2 / t2 / 1e6,
+        "roofline": {"bound": "mfma", "kernel": "grouped_gemm_nt_kernel", "achieved": (f1 + f2) / (t1 + t2) / 1e6,
+                     "peak": peak, "unit": "TFLOP/s", "frac": (f1 + f2) / (t1 + t2) / 1e6 / peak, "traffic": None},
+        "library_dense_gemm_TFLOPs": 2.0 * used * H * Hp / t3 / 1e6,
+    }
 
 
 def main():
@@ -420,6 +479,8 @@ def main():
                 torch.cuda.empty_cache()
         line["maxvio_sweep"] = sweep
         line["weights"] = bench_weights(args.seed, max(5, args.steps // 2))
+        torch.cuda.empty_cache()
+        line["ffn"] = bench_ffn(args.seed, max(5, args.steps // 2))
     print(json.dumps(line))
 
 

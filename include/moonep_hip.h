@@ -166,6 +166,24 @@ int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t rank_stride_e
                     const int32_t* experts_to_copy, int rank, int epn, int R,
                     int64_t elems_per_expert, void* stream);
 
+/*
+ * Expert-side consumer of the dispatched rows: grouped bf16 GEMM on the matrix
+ * cores, C = A * B[g]^T with fp32 accumulation.  No counterpart among the
+ * reference's launchers: the reference leaves the expert FFN to the caller and
+ * only fixes its contract (README.md:43-58: 2*epn groups delimited by
+ * cu_seqlens, local experts then prefetch slots).
+ *   A [M,K] bf16 rows (a rank's shard); cu_seqlens [G] padded end row of each
+ *   group (device memory, as mep_plan wrote it; every end a multiple of 128,
+ *   i.e. token_padding % 128 == 0); B [G,N,K] bf16, K contiguous; C [M,N] bf16.
+ *   swiglu == 0: C = bf16(row_scale[m] * acc), row_scale [M] fp32 or NULL;
+ *   swiglu != 0: C = bf16(silu(A*B[g]^T) * (A*B_up[g]^T)), B_up [G,N,K].
+ * Rows at or beyond cu_seqlens[G-1] are not written.
+ * M % 128 == 0, K % 64 == 0, N % 256 == 0 (N % 128 == 0 with swiglu).
+ */
+int mep_grouped_gemm_nt(const void* A, const void* B, const void* B_up, const int32_t* cu_seqlens,
+                        int G, void* C, const float* row_scale, int M, int N, int K, int swiglu,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

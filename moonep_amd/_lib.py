@@ -45,6 +45,7 @@ _SIGNATURES = {
     "mep_prefetch": (_i, [_i, C.POINTER(_p), C.POINTER(_p), C.POINTER(_i64), C.POINTER(_i64),
                           _p, _i, _i, _i, _p]),
     "mep_grad_reduce": (_i, [_p, _p, _i64, _p, _i, _i, _i, _i64, _p]),
+    "mep_grouped_gemm_nt": (_i, [_p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)

@@ -15,7 +15,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmoonep_hip.so")
-SOURCES = ["capi.hip", "planner.hip", "dispatch.hip", "combine.hip", "prefetch.hip"]
+SOURCES = ["capi.hip", "planner.hip", "dispatch.hip", "combine.hip", "prefetch.hip",
+           "grouped_gemm.hip"]
 FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",
     "-Wall", "-Wno-unused-function",

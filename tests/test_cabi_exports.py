@@ -90,3 +90,10 @@ def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
     assert lib.mep_grad_reduce(A, A, 16 * 4, A, 0, 4, 2, 18, None) == -2                   # elems % 4 != 0
     assert lib.mep_grad_reduce(A, A, 8, A, 0, 4, 2, 16, None) == -1                        # stride too small
     assert lib.mep_grad_reduce(A + 4, A, 64, A, 0, 4, 2, 16, None) == -4
+    # grouped GEMM: tile multiples, swiglu needs the up weights and no row scale
+    assert lib.mep_grouped_gemm_nt(A, A, None, A, 4, A, None, 100, 256, 64, 0, None) == -2
+    assert lib.mep_grouped_gemm_nt(A, A, None, A, 4, A, None, 128, 128, 64, 0, None) == -2
+    assert lib.mep_grouped_gemm_nt(A, A, None, A, 4, A, None, 128, 256, 32, 0, None) == -2
+    assert lib.mep_grouped_gemm_nt(A, A, None, A, 4, A, None, 128, 128, 64, 1, None) == -1
+    assert lib.mep_grouped_gemm_nt(A, A, A, A, 4, A, A, 128, 128, 64, 1, None) == -1
+    assert lib.mep_grouped_gemm_nt(A + 8, A, None, A, 4, A, None, 128, 256, 64, 0, None) == -4
