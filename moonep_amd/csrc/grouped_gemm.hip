@@ -4,12 +4,13 @@
 // group g multiplies by its own weight matrix B[g] stored [N,K] (K
 // contiguous), so C = A * B[g]^T needs no transposition on either operand.
 //
-// Workgroup: 512 threads, a 128 x 256 tile of (rows x weight rows), K in
-// steps of 64 through double-buffered LDS; each of the 8 waves owns 64 x 64 of
-// the tile as 2 x 2 MFMA 32x32x16 accumulators.  With token_padding a
-// multiple of 128 a row tile never straddles two groups.  The wide weight
-// tile is what the kernel's rate hangs on: it is bound by L2 -> LDS traffic
-// (a 128 x 128 tile reached 0.7 PFLOP/s at 11 TB/s of tile loads).
+// Workgroup: 640 threads on a 128 x 256 tile of (rows x weight rows), K in
+// steps of 64: two producer waves stream the tile slices from global memory
+// straight into a ring of three LDS stages, eight consumer waves own 64 x 64
+// of the tile each as 2 x 2 MFMA 32x32x16 accumulators.  With token_padding a
+// multiple of 128 a row tile never straddles two groups.  The kernel is bound
+// by the L2 (its channels are ~75 % busy at 0.8 PFLOP/s), i.e. by tile bytes
+// per flop.
 // Two epilogues:
 //   scale  : C[m,n] = bf16(row_scale[m] * acc)               (down projection)
 //   swiglu : C[m,n] = bf16(silu(A*Bg^T) * (A*Bu^T))           (gate/up fused;
@@ -26,10 +27,16 @@ typedef __bf16 mep_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float mep_f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kBM = 128, kBN = 256, kBK = 64;  // rows, weight rows, K per step of a tile
-constexpr int kPitch = kBK * 2 + 16;  // bytes per LDS row: 8 lanes of a 16-byte read hit 32 distinct banks
-constexpr int kATile = kBM * kPitch, kBTile = kBN * kPitch;
-constexpr int kGemmThreads = 512;
+constexpr int kRowBytes = kBK * 2;             // an LDS row is one 128-byte slice, no padding
+constexpr int kATile = kBM * kRowBytes, kBTile = kBN * kRowBytes;
+constexpr int kStage = kATile + kBTile;        // 48 KB
+constexpr int kStages = 3;
+constexpr int kConsumers = 8, kProducers = 2;  // waves
+constexpr int kGemmThreads = (kConsumers + kProducers) * 64;
 constexpr int kPanel = 8;  // row tiles that share a sweep over the weight tiles
+// 1 KB pieces (8 rows x 128 bytes) of a stage that one producer wave moves per step
+constexpr int kPiecesPerProducer = (kBM + kBN) / 8 / kProducers;  // 24
+static_assert(2 * kPiecesPerProducer < 64, "two steps of loads must fit the 6-bit load counter");
 
 struct GemmArgs {
   const uint16_t* A;   // [M,K]
@@ -43,21 +50,32 @@ struct GemmArgs {
 
 __device__ __forceinline__ float mep_silu(float x) { return x / (1.0f + __expf(-x)); }
 
+// s_waitcnt vmcnt(n) alone (expcnt and lgkmcnt left at "do not wait")
+template <int N>
+__device__ __forceinline__ void mep_wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// Producer / consumer waves.  Two producer waves stream the tiles from global
+// memory straight into a ring of three LDS stages (global_load_lds, 16 bytes
+// per lane: no registers, no LDS store instructions), always two K steps
+// ahead; eight consumer waves only read LDS and feed the matrix cores.  One
+// s_barrier per K step hands a filled stage to the consumers and a drained one
+// back to the producers.  A stage row is the bare 128-byte slice; the 16-byte
+// vector q of row r sits at position q ^ (r & 7), so the eight rows a group of
+// eight lanes reads fall into distinct banks.
 template <bool SWIGLU>
 __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char gsm[];
+  extern __shared__ __attribute__((aligned(1024))) char gsm[];
   __shared__ int s_group;
-  char* As = gsm;                // [2][kBM][kPitch]
-  char* Bs = gsm + 2 * kATile;   // [2][kBN][kPitch]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave & 1, wn = wave >> 1;  // 2 x 4 waves, 64 x 64 each
 
   // ---- which tile: XCD x (workgroups x, x+8, ...) walks a contiguous range of
   // tiles; inside a panel of kPanel row tiles the row tile index runs fastest
   const int total = a.mtiles * a.ntiles;
   const int per_xcd = (total + 7) >> 3;
   const int L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (L >= total || (int)(blockIdx.x >> 3) >= per_xcd) return;
+  if (L >= total) return;
   const int panel = L / (kPanel * a.ntiles);
   const int within = L - panel * (kPanel * a.ntiles);
   const int ph = min(kPanel, a.mtiles - panel * kPanel);
@@ -81,41 +99,52 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   const int g = s_group;
   if (g < 0) return;  // rows past the last group: nothing to compute
 
-  // ---- global -> register -> LDS staging: 8 threads read the 128 bytes of one
-  // row slice; a thread covers rows lrow + 64*i of the row tile (i < 2) and of
-  // the weight tile (i < 4)
-  const int lrow = tid >> 3, kv = tid & 7;
+  const int KT = a.K / kBK;
   const size_t K = (size_t)a.K;
-  const uint16_t* Ag = a.A + (size_t)(m0 + lrow) * K + kv * 8;
-  const uint16_t* Bg[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if (SWIGLU) {  // weight tile = kBN/2 gate rows, then the same kBN/2 up rows
-      const uint16_t* base = (i < 2 ? a.B : a.B2) + (size_t)g * a.N * K;
-      Bg[i] = base + (size_t)(n0 + lrow + 64 * (i & 1)) * K + kv * 8;
-    } else {
-      Bg[i] = a.B + (size_t)g * a.N * K + (size_t)(n0 + lrow + 64 * i) * K + kv * 8;
-    }
-  }
-  // two register sets: the loads of K step kt+2 are issued while step kt is
-  // multiplied, and staged into LDS one step later, so a load has two steps
-  // (and the other resident workgroup) to arrive
-  mep_u4 ra[2][2], rb[2][4];
-  auto load = [&](int set, int k0) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) ra[set][i] = *(const mep_u4*)(Ag + (size_t)i * 64 * K + k0);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rb[set][i] = *(const mep_u4*)(Bg[i] + k0);
-  };
-  auto stage = [&](int set, int buf) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-      *(mep_u4*)(As + buf * kATile + (lrow + 64 * i) * kPitch + kv * 16) = ra[set][i];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *(mep_u4*)(Bs + buf * kBTile + (lrow + 64 * i) * kPitch + kv * 16) = rb[set][i];
-  };
 
+  if (wave >= kConsumers) {
+    // =============================== producer ===============================
+    const int p = wave - kConsumers;
+    const int r = lane >> 3, kv = lane & 7;
+    // piece j of a stage: rows 8j .. 8j+7 of the row tile (j < 16), then of the
+    // weight tile; this wave moves the pieces j = p, p + kProducers, ...
+    // lane (r, kv) fetches vector kv ^ r of its row into slot (r, kv)
+    const uint16_t* Ap = a.A + (size_t)(m0 + r) * K + ((kv ^ r) * 8);
+    const uint16_t* Bp0 = a.B + (size_t)g * a.N * K + (size_t)(n0 + r) * K + ((kv ^ r) * 8);
+    const uint16_t* Bp1 = SWIGLU ? a.B2 + (size_t)g * a.N * K + (size_t)(n0 + r) * K + ((kv ^ r) * 8)
+                                 : Bp0 + (size_t)(kBN / 2) * K;
+    auto issue = [&](int k0, int stage) {
+      char* base = gsm + stage * kStage;
+#pragma unroll
+      for (int q = 0; q < kPiecesPerProducer; ++q) {
+        const int j = p + q * kProducers;  // 0 .. 47
+        const uint16_t* src;
+        if (j < kBM / 8) src = Ap + (size_t)(8 * j) * K + k0;
+        else if (j < kBM / 8 + kBN / 16) src = Bp0 + (size_t)(8 * (j - kBM / 8)) * K + k0;
+        else src = Bp1 + (size_t)(8 * (j - kBM / 8 - kBN / 16)) * K + k0;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)(base + j * 1024),
+                                         16, 0, 0);
+      }
+    };
+    const int klast = (KT - 1) * kBK;
+    issue(0, 0);
+    issue(min(kBK, klast), 1);
+    mep_wait_vmcnt<kPiecesPerProducer>();  // step 0 has landed
+    __builtin_amdgcn_s_barrier();
+    int st = 2;  // stage of step kt + 2
+    for (int kt = 0; kt < KT; ++kt) {
+      issue(min((kt + 2) * kBK, klast), st);
+      st = st == kStages - 1 ? 0 : st + 1;
+      mep_wait_vmcnt<kPiecesPerProducer>();  // everything up to step kt + 1 has landed
+      __builtin_amdgcn_s_barrier();
+    }
+    mep_wait_vmcnt<0>();
+    return;
+  }
+
+  // ================================ consumer =================================
+  const int wm = wave & 1, wn = wave >> 1;  // 2 x 4 waves, 64 x 64 each
   mep_f32x16 acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -124,50 +153,37 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  // operand rows of this lane inside the LDS tiles
+  // operand rows of this lane inside a stage (weight rows follow the kBM rows)
   const int arow = 64 * wm + (lane & 31);
-  const int brow0 = SWIGLU ? 32 * wn + (lane & 31) : 64 * wn + (lane & 31);
-  const int brow1 = SWIGLU ? kBN / 2 + 32 * wn + (lane & 31) : brow0 + 32;
-  const int koff = (lane >> 5) * 16;
+  const int brow0 = kBM + (SWIGLU ? 32 * wn + (lane & 31) : 64 * wn + (lane & 31));
+  const int brow1 = SWIGLU ? brow0 + kBN / 2 : brow0 + 32;
+  const int sw = lane & 7;      // (row & 7) of every operand row of this lane
+  const int half = lane >> 5;   // which 8 of the 16 K values of an MFMA step
+  const int oa0 = arow * kRowBytes, oa1 = (arow + 32) * kRowBytes;
+  const int ob0 = brow0 * kRowBytes, ob1 = brow1 * kRowBytes;
 
-  const int KT = a.K / kBK;
-  auto multiply = [&](int cur, int ks0, int ks1) {
-    const char* Ab = As + cur * kATile;
-    const char* Bb = Bs + cur * kBTile;
+  __builtin_amdgcn_s_barrier();  // stage 0 is filled
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  int st = 0;
+  for (int kt = 0; kt < KT; ++kt) {
+    const char* sb = gsm + st * kStage;
 #pragma unroll
-    for (int ks = ks0; ks < ks1; ++ks) {
-      const mep_bf16x8 a0 = *(const mep_bf16x8*)(Ab + arow * kPitch + ks * 32 + koff);
-      const mep_bf16x8 a1 = *(const mep_bf16x8*)(Ab + (arow + 32) * kPitch + ks * 32 + koff);
-      const mep_bf16x8 b0 = *(const mep_bf16x8*)(Bb + brow0 * kPitch + ks * 32 + koff);
-      const mep_bf16x8 b1 = *(const mep_bf16x8*)(Bb + brow1 * kPitch + ks * 32 + koff);
+    for (int ks = 0; ks < kBK / 16; ++ks) {
+      const int col = ((2 * ks + half) ^ sw) * 16;
+      const mep_bf16x8 a0 = *(const mep_bf16x8*)(sb + oa0 + col);
+      const mep_bf16x8 a1 = *(const mep_bf16x8*)(sb + oa1 + col);
+      const mep_bf16x8 b0 = *(const mep_bf16x8*)(sb + ob0 + col);
+      const mep_bf16x8 b1 = *(const mep_bf16x8*)(sb + ob1 + col);
       acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
       acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
       acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
       acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[1][1], 0, 0, 0);
     }
-  };
-  // Loads and stagings are unconditional (steps past the end re-read the last
-  // slice): a load behind a branch would force the compiler to wait for every
-  // outstanding load before staging, which empties the pipeline.
-  const int klast = (KT - 1) * kBK;
-  load(0, 0);
-  load(1, min(kBK, klast));
-  stage(0, 0);
-  __syncthreads();
-  int kt = 0;
-  for (; kt + 1 < KT; kt += 2) {  // buffer 0 holds step kt, register set 1 step kt+1
-    load(0, min((kt + 2) * kBK, klast));
-    multiply(0, 0, 2);
-    stage(1, 1);  // in the middle of the step: the LDS writes hide behind other waves' MFMAs
-    multiply(0, 2, 4);
-    __syncthreads();
-    load(1, min((kt + 3) * kBK, klast));
-    multiply(1, 0, 2);
-    stage(0, 0);
-    multiply(1, 2, 4);
-    __syncthreads();
+    st = st == kStages - 1 ? 0 : st + 1;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the reads of this stage are done
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   }
-  if (kt < KT) multiply(0, 0, 4);  // odd number of steps
 
   // ---- epilogue.  acc[i][j][v]: row 64*wm + 32*i + 8*(v/4) + 4*(lane/32) + v%4,
   // column (lane % 32) of the j-th 32-wide block
@@ -179,8 +195,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
       const int m = m0 + 64 * wm + 32 * i + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
       if (SWIGLU) {
         const int n = n0 + 32 * wn + (lane & 31);
-        const float r = mep_silu(acc[i][0][v]) * acc[i][1][v];
-        a.C[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(r);
+        const float res = mep_silu(acc[i][0][v]) * acc[i][1][v];
+        a.C[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(res);
       } else {
         const float sc = a.scale ? a.scale[m] : 1.0f;
 #pragma unroll
@@ -214,9 +230,9 @@ extern "C" int mep_grouped_gemm_nt(const void* A, const void* B, const void* B_u
   const int64_t total = (int64_t)a.mtiles * a.ntiles;
   MEP_REQUIRE(total < (1 << 30), MEP_ERR_UNSUPPORTED);
   const int per_xcd = (int)((total + 7) / 8);
-  const size_t lds = 2 * (size_t)(kATile + kBTile);
+  const size_t lds = (size_t)kStages * kStage;
   hipStream_t st = (hipStream_t)stream;
-  {  // 108 KB of dynamic LDS needs the opt-in, once per device
+  {  // 144 KB of dynamic LDS needs the opt-in, once per device
     static std::atomic<uint64_t> opted{0};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
