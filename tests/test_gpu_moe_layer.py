@@ -75,3 +75,59 @@ def test_moe_layer_forward_backward_matches_dense(cuda, sigma):
     used = tpe.sum(0).reshape(R, epn) > 0
     assert bool(((got["m0"].abs().amax(dim=(2, 3)) > 0).cpu() == used).all())
     group.destroy()
+
+
+def test_moe_layer_forward_on_hip_kernels_only(cuda):
+    """The same layer, forward only, with every step a HIP kernel of this
+    library: dispatch -> prefetch -> grouped MFMA FFN (cu_seqlens stay on the
+    device) -> combine.  One rank's chain is also captured in a HIP graph and
+    replayed.  Compared with the dense reference at the same bf16 tolerance."""
+    from moonep_amd.ffn import grouped_ffn_hip
+    from moonep_amd.prefetch import launch_prefetch
+
+    R, epn, S, K, H, Hp, tp = 4, 2, 40, 3, 256, 128, 128
+    E = R * epn
+    topk = torch.stack([routing.popularity_biased(S, K, E, R, r, 2.0, seed=9) for r in range(R)])
+    tpe = routing.tokens_per_expert(topk, E)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(R, S, H, generator=g).to(cuda)
+    w = torch.softmax(torch.randn(R, S, K, generator=g), -1).to(cuda)
+    master = [(torch.randn(R, epn, H, Hp, generator=g) * 0.08).to(cuda) for _ in range(3)]
+    topk_d, tpe_d = topk.to(cuda), tpe.to(cuda)
+
+    group = moe.EmulatedGroup(S, H, K, E, R, token_padding=tp)
+    with torch.no_grad():
+        rows, slots, cu, plans = moe.group_dispatch(group, x.to(torch.bfloat16), w, topk_d, tpe_d)
+        etc = plans[0].experts_to_copy
+        assert bool((etc >= 0).any()), "the skewed routing must exercise prefetch slots"
+        # compute views, K-contiguous: gate/up [R, 2*epn, H', H], down [R, 2*epn, H, H']
+        local = [master[0].transpose(2, 3).contiguous().to(torch.bfloat16),
+                 master[1].transpose(2, 3).contiguous().to(torch.bfloat16),
+                 master[2].to(torch.bfloat16).contiguous()]
+        pools = [torch.zeros_like(t) for t in local]
+        for r in range(R):
+            launch_prefetch(tuple(t[r] for t in local), tuple(pools), etc, rank=r)
+        views = [torch.cat([l, p], dim=1) for l, p in zip(local, pools)]
+        y = torch.stack([grouped_ffn_hip(rows[r].contiguous(), slots[r].contiguous(), cu[r].contiguous(),
+                                         views[0][r], views[1][r], views[2][r]) for r in range(R)])
+        out = moe.group_combine(group, plans, y)
+        ref = _dense_reference(x, w, topk_d, master, epn)
+        torch.cuda.synchronize()
+    err = float((out.float() - ref).abs().max())
+    scale = float(ref.abs().max())
+    assert err <= 0.03 * scale + 1e-6, (err, scale)
+    cos = float(torch.nn.functional.cosine_similarity(out.float().flatten(), ref.flatten(), dim=0))
+    assert cos > 0.999, cos
+
+    # rank 0's FFN under a HIP graph: cu_seqlens are read by the kernel, not by the host
+    r0 = (rows[0].contiguous(), slots[0].contiguous(), cu[0].contiguous())
+    eager = grouped_ffn_hip(*r0, views[0][0], views[1][0], views[2][0])
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = grouped_ffn_hip(*r0, views[0][0], views[1][0], views[2][0])
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured.view(torch.int16), eager.view(torch.int16))
+    group.destroy()
