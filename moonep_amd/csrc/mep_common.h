@@ -159,6 +159,12 @@ __device__ __forceinline__ mep_u4 mep_ld16(const void* p) {
 __device__ __forceinline__ void mep_st16_stream(void* p, mep_u4 v) {
   __builtin_nontemporal_store(v, (mep_u4*)p);
 }
+// Store written through at system scope (sc0 sc1).  For long contiguous copy
+// streams it measured up to 19 % faster than the nontemporal hint (expert
+// weight prefetch); for scattered rows (dispatch, combine) it is no better.
+__device__ __forceinline__ void mep_st16_through(void* p, mep_u4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
+}
 __device__ __forceinline__ void mep_st16(void* p, mep_u4 v) {
   *(mep_u4*)p = v;
 }

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kBlock) void prefetch_kernel(PrefetchArgs a) {
 #pragma unroll
         for (int i = 0; i < kVecPerThread; ++i) {
           const int64_t o = ((int64_t)i * kBlock + threadIdx.x) * 16;
-          if (in[i]) mep_st16_stream(dstp + o, v[i]);
+          if (in[i]) mep_st16_through(dstp + o, v[i]);
         }
       }
     }
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
 #pragma unroll
     for (int i = 0; i < kVecPerThread; ++i) {
       const int64_t o = (int64_t)i * kBlock + threadIdx.x;
-      if (in[i]) g[o] = acc[i];
+      if (in[i]) mep_st16_through(g + o, __builtin_bit_cast(mep_u4, acc[i]));
     }
   }
 }
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(kBlock) void grad_clear_kernel(ReduceArgs a) {
 #pragma unroll
     for (int i = 0; i < kVecPerThread; ++i) {
       const int64_t o = (int64_t)i * kBlock + threadIdx.x;
-      if (tile * kTileVecs + o < vecs) __builtin_nontemporal_store(zero, p + o);
+      if (tile * kTileVecs + o < vecs) mep_st16_through(p + o, __builtin_bit_cast(mep_u4, zero));
     }
   }
 }
