@@ -99,3 +99,32 @@ def test_grouped_ffn_matches_the_torch_consumer(cuda):
     scale = want.float().abs().amax(dim=1, keepdim=True).clamp(min=1e-6)
     assert float((err / scale).max()) < 0.03
     assert (got[int(ends[-1]):] == 0).all()
+
+
+def test_grouped_gemm_at_the_real_shape(cuda):
+    """One rank's shard at the headline shape (NvS = 40960 rows, H = 7168,
+    H' = 2048, 64 groups of uneven size): the fused SwiGLU GEMM is bit-identical
+    from launch to launch, and three groups (first, middle, last) match the fp32
+    reference."""
+    M, H, Hp, G = 40960, 7168, 2048, 64
+    sizes = 384 + 128 * (torch.arange(G) % 4)            # 384 .. 768 rows per group
+    ends = sizes.cumsum(0).to(torch.int32).to(cuda)
+    assert int(ends[-1]) <= M
+    g = torch.Generator(device=cuda).manual_seed(3)
+    rows = torch.randn(M, H, device=cuda, generator=g).to(torch.bfloat16)
+    gate = (torch.randn(G, Hp, H, device=cuda, generator=g) * 0.02).to(torch.bfloat16)
+    up = (torch.randn(G, Hp, H, device=cuda, generator=g) * 0.02).to(torch.bfloat16)
+    first = launch_grouped_gemm_nt(rows, gate, ends, up_weights=up)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        again = launch_grouped_gemm_nt(rows, gate, ends, up_weights=up)
+        torch.cuda.synchronize()
+        assert torch.equal(first.view(torch.int16), again.view(torch.int16))
+    start = 0
+    for gi, end in enumerate(ends.tolist()):
+        if gi in (0, G // 2, G - 1):
+            x = rows[start:end].float()
+            want = torch.nn.functional.silu(x @ gate[gi].float().t()) * (x @ up[gi].float().t())
+            _close(first[start:end].cpu(), want.cpu(), f"group {gi}")
+        start = end
+    assert (first[int(ends[-1]):] == 0).all()
