@@ -83,6 +83,20 @@ int mep_plan(const int32_t* tpe_RE, const int32_t* topk_SK, int rank, int S, int
              void* scratch, size_t scratch_bytes, void* stream);
 
 /*
+ * mep_plan that also warms the last-level cache.  No counterpart in the
+ * reference: the planner is latency-bound and occupies a few CUs; the other
+ * CUs meanwhile read the `warm_bytes` at `warm` (16-byte aligned; the token
+ * rows the following mep_dispatch copies) once, so that dispatch reads them
+ * from cache instead of mixing HBM reads into its write stream.  warm == NULL
+ * is mep_plan.
+ */
+int mep_plan_warm(const int32_t* tpe_RE, const int32_t* topk_SK, int rank, int S, int K, int E,
+                  int R, int token_padding, int NvS, int32_t* dst, int32_t* cu_seqlens,
+                  int32_t* experts_to_copy, int32_t* zero_fill, int32_t* remote_stats,
+                  void* scratch, size_t scratch_bytes, const void* warm, size_t warm_bytes,
+                  void* stream);
+
+/*
  * The same planner for ranks rank0 .. rank0+nranks-1 in one launch (one GPU
  * standing in for several ranks).  topk is [nranks,S,K]; dst, cu_seqlens,
  * zero_fill and remote_stats gain a leading [nranks] dimension;

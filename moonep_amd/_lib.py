@@ -34,6 +34,7 @@ _SIGNATURES = {
     "mep_strerror": (C.c_char_p, [_i]),
     "mep_plan_scratch_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "mep_plan": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "mep_plan_warm": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p, _sz, _p]),
     "mep_plan_ranks": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),
     "mep_dispatch": (_i, [_p, _p, _p, _p, _p, _i64, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _i,
                           C.c_uint, _p]),

@@ -318,7 +318,7 @@ class Buffer:
                 plan.zero_fill_ranges.copy_(zfr[r])
                 plan.remote_stats.copy_(stats[r])
             else:
-                launch_planning(ctx, topk.reshape(-1), tpe, cu_seqlens, plan)
+                launch_planning(ctx, topk.reshape(-1), tpe, cu_seqlens, plan, warm=hidden_sh)
         launch_dispatch(ctx, hidden_sh, route_weights_sk, plan,
                         build_dedup_map=planning_args is not None, write_dups=True,
                         dst_all_ranks=dst_all, pdl_trigger=self.enable_pdl)

@@ -26,6 +26,12 @@ struct PlanArgs {
   int* remote_stats; // [nranks, 2]
   int* scratch;      // alloc/base tables when they do not fit in LDS
   int rank0, S, K, E, R, epn, tp, NvS, tok_per_wg;
+  // optional: a byte range the workgroups beyond `groups` read once, so that it
+  // sits in the last-level cache when the planner is done (the tokens that the
+  // following dispatch copies); the planner itself occupies only a few CUs
+  const char* warm;
+  size_t warm_vecs;  // 16-byte vectors
+  int groups;        // workgroups per rank that plan
 };
 
 // LDS layout in ints (must match plan_lds_ints on the host)
@@ -62,13 +68,34 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   int* s_ce = s_bal + R;         // [NT] expert of each entry of my slice
   int* s_cd = s_ce + NT;         // [NT] destination rank of each entry
   int* tbl = kLdsTables ? (s_cd + NT)
-                        : a.scratch + (size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 2 * E * R;
+                        : a.scratch + (size_t)(blockIdx.y * a.groups + blockIdx.x) * 2 * E * R;
   int* alloc = tbl;            // [E,R] tokens of expert e landing on rank d
   int* base = tbl + E * R;     // [E,R] first slot of e on d, as an encoded dst
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  if ((int)blockIdx.x >= a.groups) {
+    // cache warmer: plain 16-byte loads, eight in flight.  The values only feed
+    // a comparison that guards a sleep, so the loads stay and nothing is written.
+    if (blockIdx.y != 0 || a.warm_vecs == 0) return;
+    const size_t nthreads = (size_t)(gridDim.x - a.groups) * NT;
+    const size_t first = (size_t)(blockIdx.x - a.groups) * NT + tid;
+    const mep_u4* w = (const mep_u4*)a.warm;
+    mep_u4 x = {0u, 0u, 0u, 0u};
+    for (size_t i = first; i < a.warm_vecs; i += 8 * nthreads) {
+      mep_u4 t[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const size_t j = i + u * nthreads;
+        t[u] = w[j < a.warm_vecs ? j : a.warm_vecs - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) x ^= t[u];
+    }
+    if ((x[0] ^ x[1]) == 0x9e3779b9u && (x[2] ^ x[3]) == 0x7f4a7c15u) __builtin_amdgcn_s_sleep(1);
+    return;
+  }
   const int rank = a.rank0 + blockIdx.y;
   const bool writer = blockIdx.x == 0;  // one workgroup per rank stores the small outputs
 
@@ -402,11 +429,11 @@ extern "C" size_t mep_plan_scratch_bytes(int S, int K, int E, int R, int nranks)
   return (size_t)c.groups * nranks * 2 * (size_t)E * R * sizeof(int);
 }
 
-extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int nranks,
-                              int S, int K, int E, int R, int token_padding, int NvS, int32_t* dst,
-                              int32_t* cu_seqlens, int32_t* experts_to_copy, int32_t* zero_fill,
-                              int32_t* remote_stats, void* scratch, size_t scratch_bytes,
-                              void* stream) {
+namespace {
+int plan_launch(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int nranks, int S, int K,
+                int E, int R, int token_padding, int NvS, int32_t* dst, int32_t* cu_seqlens,
+                int32_t* experts_to_copy, int32_t* zero_fill, int32_t* remote_stats, void* scratch,
+                size_t scratch_bytes, const void* warm, size_t warm_bytes, void* stream) {
   MEP_REQUIRE(tpe_RE && topk_nSK && dst && cu_seqlens && experts_to_copy && zero_fill &&
                   remote_stats, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(S > 0 && K > 0 && E > 0 && R > 0 && token_padding > 0 && NvS > 0, MEP_ERR_INVALID_ARG);
@@ -430,7 +457,18 @@ extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, in
   a.scratch = (int*)scratch;
   a.rank0 = rank0; a.S = S; a.K = K; a.E = E; a.R = R; a.epn = E / R; a.tp = token_padding;
   a.NvS = NvS; a.tok_per_wg = c.tok_per_wg;
-  dim3 grid(c.groups, nranks);
+  a.groups = c.groups;
+  a.warm = (const char*)warm;
+  a.warm_vecs = warm ? warm_bytes / 16 : 0;
+  // one pass of eight loads per thread covers the range; at most ~two workgroups per CU
+  int warm_groups = 0;
+  if (a.warm_vecs) {
+    const size_t per_wg = (size_t)c.nt * 8;
+    const size_t want = (a.warm_vecs + per_wg - 1) / per_wg;
+    const size_t cap = c.nt == 1024 ? 480 : 1920;
+    warm_groups = (int)(want < cap ? want : cap);
+  }
+  dim3 grid(c.groups + warm_groups, nranks);
   hipStream_t st = (hipStream_t)stream;
   if (c.nt == 1024) {
     hipLaunchKernelGGL((plan_kernel<1024, true>), grid, dim3(1024), c.lds_bytes, st, a);
@@ -454,6 +492,29 @@ extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, in
     hipLaunchKernelGGL((plan_kernel<256, false>), grid, dim3(256), c.lds_bytes, st, a);
   }
   return mep_launch_status();
+}
+
+}  // namespace
+
+extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int nranks,
+                              int S, int K, int E, int R, int token_padding, int NvS, int32_t* dst,
+                              int32_t* cu_seqlens, int32_t* experts_to_copy, int32_t* zero_fill,
+                              int32_t* remote_stats, void* scratch, size_t scratch_bytes,
+                              void* stream) {
+  return plan_launch(tpe_RE, topk_nSK, rank0, nranks, S, K, E, R, token_padding, NvS, dst, cu_seqlens,
+                     experts_to_copy, zero_fill, remote_stats, scratch, scratch_bytes, nullptr, 0,
+                     stream);
+}
+
+extern "C" int mep_plan_warm(const int32_t* tpe_RE, const int32_t* topk_SK, int rank, int S, int K,
+                             int E, int R, int token_padding, int NvS, int32_t* dst,
+                             int32_t* cu_seqlens, int32_t* experts_to_copy, int32_t* zero_fill,
+                             int32_t* remote_stats, void* scratch, size_t scratch_bytes,
+                             const void* warm, size_t warm_bytes, void* stream) {
+  MEP_REQUIRE(!warm || (uintptr_t)warm % 16 == 0, MEP_ERR_ALIGNMENT);
+  return plan_launch(tpe_RE, topk_SK, rank, 1, S, K, E, R, token_padding, NvS, dst, cu_seqlens,
+                     experts_to_copy, zero_fill, remote_stats, scratch, scratch_bytes, warm,
+                     warm_bytes, stream);
 }
 
 extern "C" int mep_plan(const int32_t* tpe_RE, const int32_t* topk_SK, int rank, int S, int K,

@@ -146,10 +146,15 @@ def plan_scratch(ctx: dict, nranks: int = 1) -> torch.Tensor | None:
     return ctx[key]
 
 
-def launch_planning(ctx: dict, topk_experts_flat, tokens_per_expert, cu_seqlens, plan) -> None:
+def launch_planning(ctx: dict, topk_experts_flat, tokens_per_expert, cu_seqlens, plan, *,
+                    warm: torch.Tensor | None = None) -> None:
     """Run the planner of ctx['rank']; writes ``plan.dst``,
     ``plan.experts_to_copy``, ``plan.zero_fill_ranges``, ``plan.remote_stats``
-    and ``cu_seqlens`` in place, asynchronously on the current stream."""
+    and ``cu_seqlens`` in place, asynchronously on the current stream.
+
+    ``warm`` (not in the reference): a contiguous tensor -- the tokens the
+    following dispatch will copy -- that the CUs the planner leaves idle read
+    once while it runs, so that dispatch finds them in the last-level cache."""
     _check_planning_outputs(ctx, cu_seqlens, plan)
     _check_dedup_encoding_bounds(ctx)
     tpe = _tpe_table(ctx, tokens_per_expert)
@@ -157,13 +162,17 @@ def launch_planning(ctx: dict, topk_experts_flat, tokens_per_expert, cu_seqlens,
     assert topk_experts_flat.numel() == plan.N
     assert topk_experts_flat.is_cuda and tpe.device == topk_experts_flat.device
     scratch = plan_scratch(ctx)
-    rc = _lib.lib().mep_plan(
+    if warm is not None:
+        assert warm.is_cuda and warm.is_contiguous() and warm.device == topk_experts_flat.device
+    rc = _lib.lib().mep_plan_warm(
         tpe.data_ptr(), topk_experts_flat.data_ptr(), int(ctx["rank"]),
         int(ctx["S"]), int(ctx["K"]), int(ctx["E"]), int(ctx["R"]),
         int(ctx["token_padding"]), int(ctx["NvS"]),
         plan.dst.data_ptr(), cu_seqlens.data_ptr(), plan.experts_to_copy.data_ptr(),
         plan.zero_fill_ranges.data_ptr(), plan.remote_stats.data_ptr(),
-        _lib.ptr(scratch), 0 if scratch is None else scratch.numel(), _lib.current_stream(),
+        _lib.ptr(scratch), 0 if scratch is None else scratch.numel(),
+        _lib.ptr(warm), 0 if warm is None else warm.numel() * warm.element_size(),
+        _lib.current_stream(),
     )
     _lib.check(rc, "mep_plan")
 

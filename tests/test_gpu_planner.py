@@ -173,3 +173,33 @@ def test_planner_random_small_shapes_match_oracle(cuda):
         checked += 1
     print(f"{checked} random shapes checked", flush=True)
     assert checked >= 80
+
+
+@pytest.mark.parametrize("S,K,E,R,tp,warm_elems", [
+    (4096, 8, 256, 8, 128, 4096 * 7168),   # the headline shape with its token rows
+    (40, 3, 8, 4, 8, 40 * 64),             # one warming workgroup, mostly clamped loads
+    (17, 2, 6, 3, 4, 7),                   # fewer than 16 bytes: nothing to warm
+    (64, 4, 4096, 8, 16, 64 * 256),        # the 256-thread planner variant with scratch tables
+])
+def test_planner_with_cache_warming_is_the_same_planner(cuda, S, K, E, R, tp, warm_elems):
+    """mep_plan_warm = mep_plan plus workgroups that only read `warm`: same
+    outputs as the oracle, and the warmed tensor is left as it was."""
+    topk = torch.stack([routing.popularity_biased(S, K, E, R, r, 1.0, seed=3) for r in range(R)])
+    tpe = routing.tokens_per_expert(topk, E)
+    gp, plans, _ = oracle_world_plan(topk.numpy(), tpe.numpy(), tp)
+    g = torch.Generator().manual_seed(1)
+    warm = torch.randn(warm_elems, generator=g).to(torch.bfloat16).to(cuda)
+    before = warm.clone()
+    rank = R - 1
+    buf = Buffer(S, 16, K, E, R, token_padding=tp, rank=rank)
+    ctx = buf._require_ctx()
+    plan, cu = allocate_planning_outputs(ctx)
+    launch_planning(ctx, topk[rank].reshape(-1).contiguous().to(cuda), tpe.to(cuda), cu, plan, warm=warm)
+    torch.cuda.synchronize()
+    assert np.array_equal(plan.dst.cpu().numpy(), plans[rank].dst)
+    assert np.array_equal(cu.cpu().numpy(), plans[rank].cu_seqlens)
+    assert np.array_equal(plan.experts_to_copy.cpu().numpy(), gp.experts_to_copy)
+    assert np.array_equal(plan.zero_fill_ranges.cpu().numpy(), plans[rank].zero_fill_ranges)
+    assert np.array_equal(plan.remote_stats.cpu().numpy(), plans[rank].remote_stats)
+    assert torch.equal(warm.view(torch.int16), before.view(torch.int16))
+    buf.destroy()
