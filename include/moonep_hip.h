@@ -87,8 +87,8 @@ int mep_plan(const int32_t* tpe_RE, const int32_t* topk_SK, int rank, int S, int
  * reference: the planner is latency-bound and occupies a few CUs; the other
  * CUs meanwhile read the `warm_bytes` at `warm` (16-byte aligned; the token
  * rows the following mep_dispatch copies) once, so that dispatch reads them
- * from cache instead of mixing HBM reads into its write stream.  warm == NULL
- * is mep_plan.
+ * from cache instead of mixing HBM reads into its write stream.  At most the
+ * first 128 MiB are read.  warm == NULL is mep_plan.
  */
 int mep_plan_warm(const int32_t* tpe_RE, const int32_t* topk_SK, int rank, int S, int K, int E,
                   int R, int token_padding, int NvS, int32_t* dst, int32_t* cu_seqlens,

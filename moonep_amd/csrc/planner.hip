@@ -459,7 +459,10 @@ int plan_launch(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int n
   a.NvS = NvS; a.tok_per_wg = c.tok_per_wg;
   a.groups = c.groups;
   a.warm = (const char*)warm;
-  a.warm_vecs = warm ? warm_bytes / 16 : 0;
+  // never more than half of the 256 MB last-level cache: beyond that the read
+  // only delays the planner and evicts itself
+  constexpr size_t kWarmMax = (size_t)128 << 20;
+  a.warm_vecs = warm ? (warm_bytes < kWarmMax ? warm_bytes : kWarmMax) / 16 : 0;
   // one pass of eight loads per thread covers the range; at most ~two workgroups per CU
   int warm_groups = 0;
   if (a.warm_vecs) {
