@@ -37,6 +37,7 @@ extern "C" {
 #define MEP_ERR_UNSUPPORTED (-2)   /* shape outside what the kernels handle        */
 #define MEP_ERR_SCRATCH (-3)       /* scratch buffer missing or too small           */
 #define MEP_ERR_ALIGNMENT (-4)     /* pointer/stride not 16-byte aligned            */
+#define MEP_ERR_STATIC_LIMIT (-5)  /* input larger than the library's fixed scratch  */
 
 /* dispatch flags */
 #define MEP_DISPATCH_WRITE_DUPS 1u /* also copy rows of negative (duplicate) entries */
@@ -134,6 +135,24 @@ size_t mep_dedup_scratch_bytes(int S, int R);
 int mep_build_dedup(const int32_t* dst_RN, int rank, int S, int K, int R, int NvS,
                     int32_t* dup_groups, int32_t* dup_loffs, int32_t* dup_counts, void* scratch,
                     size_t scratch_bytes, void* stream);
+
+/*
+ * mep_build_dedup without a scratch argument and without any allocation: the
+ * builder's scratch is a fixed 1 MiB array in device memory that the library
+ * itself holds (one copy per GPU, until the process ends).  It has no
+ * counterpart in the reference; it is for callers that cannot allocate --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Same outputs as mep_build_dedup, bit for bit.
+ * Limit: mep_dedup_scratch_bytes(S, R) <= 1 MiB (S*R up to about 260 000
+ * tokens); larger inputs return MEP_ERR_STATIC_LIMIT and launch nothing.
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU
+ * (different streams or threads) race; order them.  The first call on a
+ * device looks the array's address up (no allocation, no launch): make it
+ * outside stream capture.
+ */
+int mep_build_dedup_static(const int32_t* dst_RN, int rank, int S, int K, int R, int NvS,
+                           int32_t* dup_groups, int32_t* dup_loffs, int32_t* dup_counts,
+                           void* stream);
 
 /* primary row -> its duplicate rows, in place on one rank's shard.
  * Replaces launch_dispatch_epilogue (reference moonep/dispatch_epilogue.py:366-415). */

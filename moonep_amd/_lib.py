@@ -40,6 +40,7 @@ _SIGNATURES = {
                           C.c_uint, _p]),
     "mep_dedup_scratch_bytes": (_sz, [_i, _i]),
     "mep_build_dedup": (_i, [_p, _i, _i, _i, _i, _i, _p, _p, _p, _p, _sz, _p]),
+    "mep_build_dedup_static": (_i, [_p, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "mep_dispatch_epilogue": (_i, [_p, _p, _p, _p, _i, _i, _p]),
     "mep_combine_prologue": (_i, [_p, _p, _p, _p, _i, _i, _p]),
     "mep_combine": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),

@@ -6,6 +6,8 @@
 // duplicate expansion.
 #include "mep_common.h"
 
+#include <atomic>
+
 namespace {
 
 constexpr int kWavesPerBlock = 4;
@@ -326,19 +328,67 @@ extern "C" size_t mep_dedup_scratch_bytes(int S, int R) {
   return (ntok + 2 * nblk) * sizeof(int);
 }
 
-extern "C" int mep_build_dedup(const int32_t* dst_RN, int rank, int S, int K, int R, int NvS,
-                               int32_t* dup_groups, int32_t* dup_loffs, int32_t* dup_counts,
-                               void* scratch, size_t scratch_bytes, void* stream) {
+namespace {
+
+// Fixed scratch of mep_build_dedup_static: per-token duplicate counts and the
+// per-workgroup sums of the three builder kernels, for callers that cannot
+// allocate.  1 MiB covers S*R up to 260 000 tokens (the headline shape needs
+// 129 KiB).  Every GPU the library runs on holds its own copy at its own
+// address until the process ends; host code must never pass the array's name
+// to a kernel (on the host it is only a handle for the symbol lookup) but the
+// address hipGetSymbolAddress returns for the current device.
+constexpr size_t kStaticDedupBytes = (size_t)1 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticDedupBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_static_scratch[kMaxDevices];  // device address per device, null = not looked up
+
+// Device address of `scratch` on the current device; looked up once per device.
+int static_scratch_ptr(void** out) {
+  int dev = 0;
+  MEP_RETURN_IF_HIP(hipGetDevice(&dev));
+  MEP_REQUIRE(dev >= 0 && dev < kMaxDevices, MEP_ERR_UNSUPPORTED);
+  void* p = g_static_scratch[dev].load(std::memory_order_acquire);
+  if (!p) {
+    MEP_RETURN_IF_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    MEP_REQUIRE(p != nullptr, MEP_ERR_SCRATCH);
+    g_static_scratch[dev].store(p, std::memory_order_release);  // racing threads store the same address
+  }
+  *out = p;
+  return MEP_OK;
+}
+
+}  // namespace
+
+extern "C" int mep_build_dedup_static(const int32_t* dst_RN, int rank, int S, int K, int R, int NvS,
+                                      int32_t* dup_groups, int32_t* dup_loffs,
+                                      int32_t* dup_counts, void* stream) {
   MEP_REQUIRE(dst_RN && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(S > 0 && K > 0 && R > 0 && NvS > 0 && rank >= 0 && rank < R, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE((int64_t)S * R < INT32_MAX, MEP_ERR_UNSUPPORTED);
-  MEP_REQUIRE(scratch && scratch_bytes >= mep_dedup_scratch_bytes(S, R), MEP_ERR_SCRATCH);
+  MEP_REQUIRE(mep_dedup_scratch_bytes(S, R) <= kStaticDedupBytes, MEP_ERR_STATIC_LIMIT);
+  void* p = nullptr;
+  const int rc = static_scratch_ptr(&p);
+  if (rc != MEP_OK) return rc;
+  // Nothing needs clearing: the three kernels write every word of the scratch
+  // they later read (tok_dups[0, S*R), blk_sums[0, 2*nblk)) within this call.
+  return mep_build_dedup(dst_RN, rank, S, K, R, NvS, dup_groups, dup_loffs, dup_counts, p,
+                         kStaticDedupBytes, stream);
+}
+
+extern "C" int mep_build_dedup(const int32_t* dst_RN, int rank, int S, int K, int R, int NvS,
+                               int32_t* dup_groups, int32_t* dup_loffs, int32_t* dup_counts,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  MEP_REQUIRE(dst_RN && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(S > 0 && K > 0 && R > 0 && NvS > 0 && rank >= 0 && rank < R, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE((int64_t)S * R < INT32_MAX, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(workspace && workspace_bytes >= mep_dedup_scratch_bytes(S, R), MEP_ERR_SCRATCH);
   DedupArgs a;
   a.dst = dst_RN; a.dup_groups = dup_groups; a.dup_loffs = dup_loffs; a.dup_counts = dup_counts;
   a.rank = rank; a.S = S; a.K = K; a.R = R; a.NvS = NvS;
   a.ntok = S * R;
   a.nblk = (a.ntok + kDedupBlock - 1) / kDedupBlock;
-  a.tok_dups = (int*)scratch;
+  a.tok_dups = (int*)workspace;
   a.blk_sums = a.tok_dups + a.ntok;
   hipStream_t st = (hipStream_t)stream;
   hipLaunchKernelGGL(dedup_count_kernel, dim3(a.nblk), dim3(kDedupBlock), 0, st, a);

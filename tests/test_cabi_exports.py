@@ -31,7 +31,7 @@ def test_version_and_error_strings():
     lib = _lib.lib()
     assert lib.mep_version() >= 100
     assert lib.mep_strerror(0) == b"ok"
-    for code in (-1, -2, -3, -4):
+    for code in (-1, -2, -3, -4, -5):
         assert len(lib.mep_strerror(code)) > 3
 
 
@@ -98,3 +98,15 @@ def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
     assert lib.mep_grouped_gemm_nt(A, A, None, A, 4, A, None, 128, 128, 64, 1, None) == -1
     assert lib.mep_grouped_gemm_nt(A, A, A, A, 4, A, A, 128, 128, 64, 1, None) == -1
     assert lib.mep_grouped_gemm_nt(A + 8, A, None, A, 4, A, None, 128, 256, 64, 0, None) == -4
+
+
+def test_static_scratch_entry_point_rejects_inputs_beyond_its_fixed_size():
+    """mep_build_dedup_static allocates nothing: its scratch is a fixed 1 MiB device
+    array; a larger input is refused with its own error code before any device call."""
+    lib = _lib.lib()
+    A = 0x10000
+    assert lib.mep_dedup_scratch_bytes(4096, 8) <= (1 << 20)     # the headline shape fits
+    assert lib.mep_dedup_scratch_bytes(37500, 8) > (1 << 20)     # 300 000 tokens do not
+    assert lib.mep_build_dedup_static(A, 0, 37500, 8, 8, 37500 * 8 + 8192, A, A, A, None) == -5
+    assert lib.mep_build_dedup_static(None, 0, 64, 8, 8, 1024, A, A, A, None) == -1
+    assert b"fixed scratch" in lib.mep_strerror(-5)
