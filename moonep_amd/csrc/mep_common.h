@@ -162,8 +162,13 @@ __device__ __forceinline__ void mep_st16_stream(void* p, mep_u4 v) {
 // Store written through at system scope (sc0 sc1).  For long contiguous copy
 // streams it measured up to 19 % faster than the nontemporal hint (expert
 // weight prefetch); for scattered rows (dispatch, combine) it is no better.
+// The s_nop belongs to the store: a store of more than 64 bits reads its data
+// registers a few cycles after it issues, and the compiler, which cannot see
+// into the asm, would otherwise be free to overwrite them with the very next
+// VALU instruction (seen: an address computation landing in v[2:3] of a zero
+// vector one instruction after the store, leaving address bits in memory).
 __device__ __forceinline__ void mep_st16_through(void* p, mep_u4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 3" : : "v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ void mep_st16(void* p, mep_u4 v) {
   *(mep_u4*)p = v;

@@ -2,11 +2,14 @@
 //   prefetch    -- every owned expert that some rank hosts remotely is read
 //                  once and streamed to each requesting (rank, slot);
 //   grad reduce -- the fp32 grads accumulated in those slots are summed back
-//                  into the owner's grad in (rank, slot) order, then the
-//                  rank's own slots are cleared.
+//                  into the owner's grad in (rank, slot) order, and the rank's
+//                  own occupied slots are cleared, all in one launch.
 // Both are flat 16-byte-vector streaming kernels over a slot table that each
 // workgroup rebuilds in LDS from experts_to_copy (a few hundred ints), so no
 // host round trip and no second launch is needed to learn the work list.
+// Whole tiles take a path without per-vector conditions: a load behind a
+// branch makes the compiler wait for every outstanding load first, which
+// serialises a thread's loads.
 #include "mep_common.h"
 
 namespace {
@@ -81,20 +84,23 @@ struct SlotTable {
   }
 };
 
-size_t slot_table_bytes(int R, int epn) {
-  return ((size_t)2 * R * epn + 3 * (size_t)epn + 4) * sizeof(int);
-}
+__host__ __device__ inline int slot_table_ints(int R, int epn) { return 2 * R * epn + 3 * epn + 4; }
+
+size_t slot_table_bytes(int R, int epn) { return (size_t)slot_table_ints(R, epn) * sizeof(int); }
 
 // Persistent workgroups, each moving a 16 KiB tile per step.  More workgroups
-// stream a little faster (6.3 vs 5.9 TB/s at 32768 vs 2048 for a dense slot
-// table) but each pays the table set-up, which dominates when only a few
-// experts are hosted remotely -- the common case; 4096 balances the two.
-// The number of active experts is only known on the device, so the grid is
-// sized from the tiles of ONE expert: with `tiles` (or an even fraction of
-// them) workgroups every workgroup moves the same number of tiles whatever
-// that number is; small tensors spread over up to `epn` experts' tiles.
-int stream_blocks(int64_t tiles, int R, int epn) {
-  const int64_t cap = (int64_t)R * epn <= 1024 ? 4096 : 2048;
+// stream a dense slot table a little faster, but each pays the table set-up,
+// which dominates when only a few experts are hosted remotely -- the common
+// case; `cap` balances the two.  Measured at [32, 7168, 2048] per rank: the copy
+// is fastest with one workgroup per tile of an expert (1792; cap 4096), the
+// reduction with two workgroups per CU (cap 512: 5.5 TB/s on a table with 8
+// slots per rank against 4.9-5.2 with 896 to 3584 workgroups).  The number of
+// active experts is only known on the device, so the grid is sized from the
+// tiles of ONE expert: with `tiles` (or an even fraction of them) workgroups
+// every workgroup moves the same number of tiles whatever that number is; small
+// tensors spread over up to `epn` experts' tiles.
+int stream_blocks(int64_t tiles, int R, int epn, int64_t cap) {
+  if ((int64_t)R * epn > 1024 && cap > 2048) cap = 2048;  // large tables: set-up costs more
   if (tiles <= 0) return 1;
   if (8 * tiles > cap) {
     const int64_t per_block = (tiles + cap - 1) / cap;  // tiles of an expert per workgroup
@@ -130,7 +136,22 @@ __global__ __launch_bounds__(kBlock) void prefetch_kernel(PrefetchArgs a) {
       const int le = t.active[ai];
       const int64_t boff = tile * kTileBytes;
       const char* src = a.local[ti] + (int64_t)le * bytes + boff;
+      const int beg = t.off[le], end = t.off[le + 1];
       mep_u4 v[kVecPerThread];
+      if (boff + kTileBytes <= bytes) {  // whole tile: a workgroup-uniform test
+#pragma unroll
+        for (int i = 0; i < kVecPerThread; ++i)
+          v[i] = mep_ld16_stream(src + ((int64_t)i * kBlock + threadIdx.x) * 16);
+        for (int sidx = beg; sidx < end; ++sidx) {
+          const int rb = t.list[sidx];
+          const int d = rb / a.epn, b = rb - d * a.epn;
+          char* dstp = a.pool[ti] + (int64_t)d * a.rank_stride[ti] + (int64_t)b * bytes + boff;
+#pragma unroll
+          for (int i = 0; i < kVecPerThread; ++i)
+            mep_st16_through(dstp + ((int64_t)i * kBlock + threadIdx.x) * 16, v[i]);
+        }
+        continue;
+      }
       bool in[kVecPerThread];
 #pragma unroll
       for (int i = 0; i < kVecPerThread; ++i) {
@@ -138,7 +159,6 @@ __global__ __launch_bounds__(kBlock) void prefetch_kernel(PrefetchArgs a) {
         in[i] = boff + o < bytes;
         if (in[i]) v[i] = mep_ld16_stream(src + o);
       }
-      const int beg = t.off[le], end = t.off[le + 1];
       for (int sidx = beg; sidx < end; ++sidx) {
         const int rb = t.list[sidx];
         const int d = rb / a.epn, b = rb - d * a.epn;
@@ -164,23 +184,112 @@ struct ReduceArgs {
 
 typedef float mep_f4 __attribute__((ext_vector_type(4)));
 
+// zero one 16 KiB tile of slot (rank, b)
+__device__ __forceinline__ void clear_tile(const ReduceArgs& a, int b, int64_t tile, int64_t vecs) {
+  constexpr int kTileVecs = kBlock * kVecPerThread;
+  const mep_f4 zero = {0.f, 0.f, 0.f, 0.f};
+  mep_f4* p = (mep_f4*)(a.pool + (int64_t)a.rank * a.rank_stride + (int64_t)b * a.elems) +
+              tile * kTileVecs;
+#pragma unroll
+  for (int i = 0; i < kVecPerThread; ++i) {
+    const int64_t o = (int64_t)i * kBlock + threadIdx.x;
+    if (tile * kTileVecs + o < vecs) mep_st16_through(p + o, __builtin_bit_cast(mep_u4, zero));
+  }
+}
+
+// One launch does the reduction and both kinds of clears:
+//  * an own slot (a slot of `rank`) that holds one of the rank's OWN experts is
+//    in that expert's slot list; the workgroup that sums tile T of it is the
+//    only reader of that tile and zeroes it once its vectors have been added;
+//  * an own slot that holds another rank's expert is never read here; its
+//    tiles are extra work items after the reduce tiles.
 __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
   extern __shared__ int smem[];
   SlotTable t;
   t.carve(smem, a.R, a.epn);
-  t.build(a.etc, a.rank, a.R, a.epn);
+  int* occ = smem + slot_table_ints(a.R, a.epn);  // [epn] own slots holding foreign experts, [1] their number
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    const int lo = a.rank * a.epn;
+    int n = 0;
+    for (int c = 0; c < a.epn; c += 64) {
+      const int b = c + lane;
+      const int e = b < a.epn ? a.etc[a.rank * a.epn + b] : -1;
+      const bool foreign = e >= 0 && (unsigned)(e - lo) >= (unsigned)a.epn;
+      const uint64_t m = __ballot(foreign);
+      if (foreign) occ[n + __popcll(m & mep_lanes_lt())] = b;
+      n += __popcll(m);
+    }
+    if (lane == 0) occ[a.epn] = n;
+  }
+  t.build(a.etc, a.rank, a.R, a.epn);  // ends with a workgroup barrier
   const int n_active = t.misc[0];
-  if (n_active == 0) return;
+  const int n_clear = occ[a.epn];
+  if (n_active == 0 && n_clear == 0) return;
   const int64_t vecs = a.elems / 4;
   constexpr int kTileVecs = kBlock * kVecPerThread;
   const int64_t tiles = (vecs + kTileVecs - 1) / kTileVecs;
-  const int64_t work = tiles * n_active;
+  const int64_t reduce_work = tiles * n_active;
+  const int64_t work = reduce_work + tiles * n_clear;
   for (int64_t w = blockIdx.x; w < work; w += gridDim.x) {
+    if (w >= reduce_work) {
+      const int64_t c = w - reduce_work;
+      const int oi = (int)(c / tiles);
+      clear_tile(a, occ[oi], c - (int64_t)oi * tiles, vecs);
+      continue;
+    }
     const int ai = (int)(w / tiles);
     const int64_t tile = w - (int64_t)ai * tiles;
     const int le = t.active[ai];
     mep_f4* g = (mep_f4*)(a.local_grad + (int64_t)le * a.elems) + tile * kTileVecs;
+    const int beg = t.off[le], end = t.off[le + 1];
+    auto slot_ptr = [&](int sidx) -> const mep_f4* {
+      const int rb = t.list[sidx];
+      const int src = rb / a.epn, b = rb - src * a.epn;
+      return (const mep_f4*)(a.pool + (int64_t)src * a.rank_stride + (int64_t)b * a.elems) +
+             tile * kTileVecs + threadIdx.x;
+    };
+    // slot sidx belongs to `rank` itself (it then holds one of the rank's own experts)
+    auto own_slot = [&](int sidx) -> int {
+      const int rb = t.list[sidx];
+      return rb / a.epn == a.rank ? rb - a.rank * a.epn : -1;
+    };
     mep_f4 acc[kVecPerThread];
+    if ((tile + 1) * kTileVecs <= vecs) {
+      // whole tile (workgroup-uniform): unconditional loads; the vectors of the
+      // next slot are requested before those of the current one are added.  The
+      // adds stay in (source rank, slot) order.
+      mep_f4 v[kVecPerThread], nx[kVecPerThread];
+#pragma unroll
+      for (int i = 0; i < kVecPerThread; ++i) acc[i] = g[(int64_t)i * kBlock + threadIdx.x];
+      const mep_f4* p = slot_ptr(beg);
+#pragma unroll
+      for (int i = 0; i < kVecPerThread; ++i) v[i] = __builtin_nontemporal_load(p + (int64_t)i * kBlock);
+      for (int sidx = beg; sidx < end; ++sidx) {
+        const bool more = sidx + 1 < end;  // workgroup-uniform
+        if (more) {
+          const mep_f4* q = slot_ptr(sidx + 1);
+#pragma unroll
+          for (int i = 0; i < kVecPerThread; ++i)
+            nx[i] = __builtin_nontemporal_load(q + (int64_t)i * kBlock);
+        }
+#pragma unroll
+        for (int i = 0; i < kVecPerThread; ++i) acc[i] = acc[i] + v[i];
+        const int ob = own_slot(sidx);
+        if (ob >= 0) {
+          __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this slot's vectors have arrived
+          clear_tile(a, ob, tile, vecs);
+        }
+        if (more) {
+#pragma unroll
+          for (int i = 0; i < kVecPerThread; ++i) v[i] = nx[i];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kVecPerThread; ++i)
+        mep_st16_through(g + (int64_t)i * kBlock + threadIdx.x, __builtin_bit_cast(mep_u4, acc[i]));
+      continue;
+    }
     bool in[kVecPerThread];
 #pragma unroll
     for (int i = 0; i < kVecPerThread; ++i) {
@@ -188,65 +297,25 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
       in[i] = tile * kTileVecs + o < vecs;
       if (in[i]) acc[i] = g[o];
     }
-    const int beg = t.off[le], end = t.off[le + 1];
     for (int sidx = beg; sidx < end; ++sidx) {
-      const int rb = t.list[sidx];
-      const int src = rb / a.epn, b = rb - src * a.epn;
-      const mep_f4* p = (const mep_f4*)(a.pool + (int64_t)src * a.rank_stride + (int64_t)b * a.elems) +
-                        tile * kTileVecs;
+      const mep_f4* p = slot_ptr(sidx);
       mep_f4 v[kVecPerThread];
 #pragma unroll
-      for (int i = 0; i < kVecPerThread; ++i) {
-        const int64_t o = (int64_t)i * kBlock + threadIdx.x;
-        if (in[i]) v[i] = __builtin_nontemporal_load(p + o);
-      }
+      for (int i = 0; i < kVecPerThread; ++i)
+        if (in[i]) v[i] = __builtin_nontemporal_load(p + (int64_t)i * kBlock);
 #pragma unroll
       for (int i = 0; i < kVecPerThread; ++i)
         if (in[i]) acc[i] = acc[i] + v[i];
+      const int ob = own_slot(sidx);
+      if (ob >= 0) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        clear_tile(a, ob, tile, vecs);
+      }
     }
 #pragma unroll
     for (int i = 0; i < kVecPerThread; ++i) {
       const int64_t o = (int64_t)i * kBlock + threadIdx.x;
       if (in[i]) mep_st16_through(g + o, __builtin_bit_cast(mep_u4, acc[i]));
-    }
-  }
-}
-
-// zero this rank's own slots that hold any expert
-__global__ __launch_bounds__(kBlock) void grad_clear_kernel(ReduceArgs a) {
-  extern __shared__ int smem[];  // [epn] occupied slots, [1] their number
-  int* occ = smem;
-  int* nocc = smem + a.epn;
-  if (threadIdx.x < 64) {
-    const int lane = threadIdx.x;
-    int n = 0;
-    for (int c = 0; c < a.epn; c += 64) {
-      const int b = c + lane;
-      const bool used = b < a.epn && a.etc[a.rank * a.epn + b] >= 0;
-      const uint64_t m = __ballot(used);
-      if (used) occ[n + __popcll(m & mep_lanes_lt())] = b;
-      n += __popcll(m);
-    }
-    if (lane == 0) *nocc = n;
-  }
-  __syncthreads();
-  const int n_occ = *nocc;
-  if (n_occ == 0) return;
-  const int64_t vecs = a.elems / 4;
-  constexpr int kTileVecs = kBlock * kVecPerThread;
-  const int64_t tiles = (vecs + kTileVecs - 1) / kTileVecs;
-  const int64_t work = tiles * n_occ;
-  const mep_f4 zero = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t w = blockIdx.x; w < work; w += gridDim.x) {
-    const int oi = (int)(w / tiles);
-    const int b = occ[oi];
-    const int64_t tile = w - (int64_t)oi * tiles;
-    mep_f4* p = (mep_f4*)(a.pool + (int64_t)a.rank * a.rank_stride + (int64_t)b * a.elems) +
-                tile * kTileVecs;
-#pragma unroll
-    for (int i = 0; i < kVecPerThread; ++i) {
-      const int64_t o = (int64_t)i * kBlock + threadIdx.x;
-      if (tile * kTileVecs + o < vecs) mep_st16_through(p + o, __builtin_bit_cast(mep_u4, zero));
     }
   }
 }
@@ -274,10 +343,10 @@ extern "C" int mep_prefetch(int ntensors, const void* const* local, void* const*
                     (uintptr_t)pool[i] % 16 == 0, MEP_ERR_ALIGNMENT);
     a.local[i] = (const char*)local[i]; a.pool[i] = (char*)pool[i];
     a.rank_stride[i] = rank_stride_bytes[i]; a.bytes[i] = bytes_per_expert[i];
-    const int64_t tiles = (bytes_per_expert[i] + kTileBytes - 1) / kTileBytes * epn;
+    const int64_t tiles = (bytes_per_expert[i] + kTileBytes - 1) / kTileBytes;  // of one expert
     if (tiles > max_tiles) max_tiles = tiles;
   }
-  const int blocks = stream_blocks(max_tiles, R, epn);
+  const int blocks = stream_blocks(max_tiles, R, epn, 4096);
   hipLaunchKernelGGL(prefetch_kernel, dim3(blocks), dim3(kBlock), lds, (hipStream_t)stream, a);
   return mep_launch_status();
 }
@@ -292,17 +361,13 @@ extern "C" int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t ra
   MEP_REQUIRE(rank_stride_elems >= elems_per_expert * epn, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(rank_stride_elems % 4 == 0 && (uintptr_t)local_grad % 16 == 0 &&
                   (uintptr_t)reduce_pool % 16 == 0, MEP_ERR_ALIGNMENT);
-  const size_t lds = slot_table_bytes(R, epn);
+  const size_t lds = slot_table_bytes(R, epn) + ((size_t)epn + 1) * sizeof(int);  // + own foreign-held slots
   MEP_REQUIRE(lds <= 64 * 1024, MEP_ERR_UNSUPPORTED);
   ReduceArgs a{local_grad, reduce_pool, rank_stride_elems, elems_per_expert, experts_to_copy,
                rank, epn, R};
   const int64_t tiles = (elems_per_expert / 4 + kBlock * kVecPerThread - 1) /
                         (kBlock * kVecPerThread);
-  const int blocks = stream_blocks(tiles, R, epn);
-  hipStream_t st = (hipStream_t)stream;
-  // two launches: the clear must not overtake reads of a slot that holds one
-  // of this rank's own experts
-  hipLaunchKernelGGL(grad_reduce_kernel, dim3(blocks), dim3(kBlock), lds, st, a);
-  hipLaunchKernelGGL(grad_clear_kernel, dim3(blocks), dim3(kBlock), (epn + 1) * sizeof(int), st, a);
+  const int blocks = stream_blocks(tiles, R, epn, 512);
+  hipLaunchKernelGGL(grad_reduce_kernel, dim3(blocks), dim3(kBlock), lds, (hipStream_t)stream, a);
   return mep_launch_status();
 }
