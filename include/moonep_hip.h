@@ -193,11 +193,17 @@ int mep_prefetch(int ntensors, const void* const* local, void* const* pool,
  * moonep/grad_reduce.py:437-543; kernel :151-389).  local_grad[le] +=
  * reduce[src][b] over the slots holding expert rank*epn+le in (src,b)
  * ascending order; then reduce[rank][b] = 0 for every b with
- * experts_to_copy[rank,b] >= 0.  elems_per_expert % 4 == 0.
+ * experts_to_copy[rank,b] >= 0.  One launch.  elems_per_expert % 4 == 0.
+ * The reference separates the two halves with a cross-rank barrier (every rank
+ * has read before any rank clears, grad_reduce.py:369-372); a caller that drives
+ * several ranks on one GPU gets the same by calling every rank with
+ * MEP_REDUCE_NO_CLEAR first and then every rank with MEP_REDUCE_CLEAR_ONLY.
  */
+#define MEP_REDUCE_NO_CLEAR 1u   /* sum only */
+#define MEP_REDUCE_CLEAR_ONLY 2u /* zero the rank's own occupied slots only */
 int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t rank_stride_elems,
                     const int32_t* experts_to_copy, int rank, int epn, int R,
-                    int64_t elems_per_expert, void* stream);
+                    int64_t elems_per_expert, unsigned flags, void* stream);
 
 /*
  * Expert-side consumer of the dispatched rows: grouped bf16 GEMM on the matrix

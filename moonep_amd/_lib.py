@@ -23,6 +23,8 @@ COMBINE_TWO_LEVEL = 2
 COMBINE_WEIGHTED = 3
 DISPATCH_WRITE_DUPS = 1
 DISPATCH_NO_ZERO_FILL = 2
+REDUCE_NO_CLEAR = 1
+REDUCE_CLEAR_ONLY = 2
 
 _p = C.c_void_p
 _i = C.c_int
@@ -46,7 +48,7 @@ _SIGNATURES = {
     "mep_combine": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "mep_prefetch": (_i, [_i, C.POINTER(_p), C.POINTER(_p), C.POINTER(_i64), C.POINTER(_i64),
                           _p, _i, _i, _i, _p]),
-    "mep_grad_reduce": (_i, [_p, _p, _i64, _p, _i, _i, _i, _i64, _p]),
+    "mep_grad_reduce": (_i, [_p, _p, _i64, _p, _i, _i, _i, _i64, C.c_uint, _p]),
     "mep_grouped_gemm_nt": (_i, [_p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _p]),
 }
 

@@ -2,51 +2,68 @@
 MI355X.
 
 Same constructor, methods, argument meaning, return tuples and assertion
-behaviour as reference moonep/api.py:430-1208, so a caller written against
-``moonep.Buffer`` runs unchanged::
+behaviour as reference moonep/api.py:430-1208::
 
-    buffer = Buffer(S, H, K, E, num_ep_ranks, token_padding=128, rank=r)
-    hidden_nvsh, w_nvs, cu_seqlens, plan = buffer.dispatch(hidden_sh, w_sk, topk_sk, tpe_RE)
+    buffer = Buffer(S, H, K, E, num_ep_ranks, token_padding=128, rank=r, world=world)
+    hidden_nvsh, w_nvs, cu_seqlens, plan = buffer.dispatch(hidden_sh, w_sk, topk_sk, tpe)
     buffer.prefetch_weight(plan=plan, local_gate_weight=..., gate_prefetch_buffer=..., ...)
     out_sh, w_sk_back, _ = buffer.combine(plan=plan, hidden_nvsh=ffn_out, route_weights_nvs=w_nvs)
     buffer.reduce_grad(plan=plan, local_gate_grad=..., gate_reduce_buffer=..., ...)
     buffer.destroy()
 
-What differs, because one GPU stands in for the R expert-parallel ranks:
+One GPU stands in for the R expert-parallel ranks.  What that changes:
 
 * the ranks' communication shards are one ``[R * NvS, H]`` tensor in local
-  HBM (plus an ``[R * meta_chunk]`` int32 tensor for the route-weight slots)
-  instead of peer-mapped symmetric memory; several Buffers of one emulated
-  group can share them through ``world=EmulatedWorld(...)``;
-* ``rank=`` says which rank this Buffer plays (default: the
+  HBM (plus an ``[R * meta_chunk]`` int32 tensor for the route-weight slots and
+  the gathered count table) instead of peer-mapped symmetric memory: an
+  ``EmulatedWorld``.  ``rank=`` says which rank a Buffer plays (default: the
   ``torch.distributed`` rank if a group is initialised, else 0);
-* ``tokens_per_expert`` is every rank's count table ``[R, E]`` (the reference
-  gathers the rows from peers inside its planner);
+* a caller written against ``moonep.Buffer`` -- per-rank ``topk_experts_sk[S, K]``
+  and ``tokens_per_expert[E]`` -- runs unchanged when every rank is driven by its
+  own host thread on a world made with ``host_threads=True``
+  (``EmulatedWorld.run_ranks`` starts them): the points where the reference
+  synchronises its ranks (count all-gather, after the row writes, before combine
+  reads, between the read and the clear of ``reduce_grad``) become thread
+  rendezvous that also order the ranks' streams, so the count table, the
+  fresh plan's duplicate groups and every shard are complete when they are read;
+* one host thread can still drive a rank (or all of them in turn) by passing
+  what the gather would have produced: ``tokens_per_expert[R, E]``, and
+  ``topk_experts_sk[R, S, K]`` when the plan's duplicate groups are wanted.
+  With per-rank ``[S, K]`` routing and no host threads the other ranks' ``dst``
+  are unknown: the plan is then marked as having no duplicate map and the
+  kernels that need one (``launch_dispatch_epilogue``, ``launch_combine_prologue``)
+  refuse it.  Several Buffers sharing a world from one thread must use
+  ``zero_copy=True``: a copy-out taken right after one rank's dispatch would
+  miss the rows the other ranks have not written yet;
 * the duplicate expansion / pre-reduction that the reference runs as separate
   destination-side kernels is folded into dispatch and combine: dispatch
   writes all K copies, combine groups and rounds exactly as the reference's
   prologue + combine pair does, so outputs are bit-identical; the standalone
   kernels stay available as ``launch_dispatch_epilogue`` /
   ``launch_combine_prologue``;
-* ``inter_rank_sync``, ``enable_pdl``, ``num_sms`` and ``comm_stream_priority``
-  are validated like the reference and otherwise have no effect (no peers; HIP
-  kernels on one stream run back to back; the kernels size their own grids;
-  all streams stay at the default priority).
+* ``inter_rank_sync`` selects whether a threaded world's rendezvous are taken;
+  ``enable_pdl``, ``num_sms`` and ``comm_stream_priority`` are validated like the
+  reference and otherwise have no effect (HIP kernels on one stream run back to
+  back; the kernels size their own grids; all streams stay at the default
+  priority).
 """
 
 from __future__ import annotations
 
 import logging
 import os
+import threading
 import warnings
+import weakref
 
 import torch
 
 from .combine import launch_combine, launch_combine_prologue  # noqa: F401
-from .dispatch import launch_build_dedup, launch_dispatch, launch_dispatch_epilogue  # noqa: F401
+from .dispatch import (check_dispatch_inputs, launch_build_dedup, launch_dispatch,  # noqa: F401
+                       launch_dispatch_epilogue)
 from .grad_reduce import launch_grad_reduce
-from .planning import (MoonEPCommPlan, allocate_planning_outputs, launch_planning,
-                       launch_planning_all_ranks)
+from .planning import (MoonEPCommPlan, allocate_launch_scratch, allocate_planning_outputs,
+                       launch_planning, launch_planning_all_ranks)
 from .prefetch import _ELEM_TYPES, launch_prefetch
 
 logger = logging.getLogger(__name__)
@@ -57,34 +74,49 @@ def _align_up(x: int, alignment: int) -> int:
 
 
 def _validate_rank_strided_pool(pool: torch.Tensor) -> int:
-    """A pool is contiguous inside each rank, ranks may be padded apart
-    (reference moonep/api.py:85-97)."""
+    """Stride (in elements) between the ranks of a pool.  Each rank's payload is
+    one contiguous block; blocks may be padded apart but not overlap, start on
+    16-byte boundaries and lie inside the storage (the checks of reference
+    moonep/api.py:85-97)."""
     assert pool.is_cuda and pool.ndim >= 2 and pool.shape[0] > 0
-    assert pool[0].is_contiguous(), "pools must be contiguous within each rank"
-    rank_numel = pool[0].numel()
-    rank_stride = int(pool.stride(0))
-    assert rank_numel > 0 and rank_stride >= rank_numel, "rank payloads must not overlap"
-    stride_bytes = rank_stride * pool.element_size()
-    assert stride_bytes % 16 == 0 and 0 < stride_bytes < (1 << 40)
+    per_rank = pool[0]
+    assert per_rank.is_contiguous(), "pools must be contiguous within each rank"
+    payload, stride = per_rank.numel(), int(pool.stride(0))
+    assert 0 < payload <= stride, "rank payloads must not overlap"
+    itemsize = pool.element_size()
+    assert 0 < stride * itemsize < (1 << 40) and (stride * itemsize) % 16 == 0
     assert pool.data_ptr() % 16 == 0, "pools must be 16-byte aligned"
-    end = pool.storage_offset() + (pool.shape[0] - 1) * rank_stride + rank_numel
-    assert end * pool.element_size() <= pool.untyped_storage().nbytes()
-    return rank_stride
+    last_elem = pool.storage_offset() + stride * (pool.shape[0] - 1) + payload
+    assert last_elem * itemsize <= pool.untyped_storage().nbytes()
+    return stride
 
 
 def _num_sms_dedup_from_env(max_sms: int) -> int:
-    raw = os.environ.get("MOONEP_NUM_SMS_DEDUP")
-    if raw is None or raw == "":
+    """CU count for the standalone duplicate kernels: ``MOONEP_NUM_SMS_DEDUP`` when
+    set (an integer in [1, max_sms]), else all of them."""
+    text = os.environ.get("MOONEP_NUM_SMS_DEDUP", "")
+    if text == "":
         return max_sms
-    try:
-        value = int(raw)
-    except ValueError as exc:
-        raise ValueError(
-            f"MOONEP_NUM_SMS_DEDUP must be an integer in [1, {max_sms}], got {raw!r}"
-        ) from exc
-    if not (1 <= value <= max_sms):
+    if not text.lstrip("+-").isdigit():
+        raise ValueError(f"MOONEP_NUM_SMS_DEDUP must be an integer in [1, {max_sms}], got {text!r}")
+    value = int(text)
+    if value < 1 or value > max_sms:
         raise ValueError(f"MOONEP_NUM_SMS_DEDUP must be in [1, {max_sms}], got {value}")
     return value
+
+
+def _check_num_sms(num_sms, max_sms: int) -> int:
+    """``num_sms`` as the reference validates it (moonep/api.py:231-248): type and
+    sign before anything touches the device, default min(32, CUs)."""
+    if num_sms is None:
+        return min(32, max_sms)
+    if isinstance(num_sms, bool) or not isinstance(num_sms, int):
+        raise TypeError(f"num_sms must be a positive int, got {type(num_sms).__name__}")
+    if num_sms < 1:
+        raise ValueError(f"num_sms must be a positive int, got {num_sms}")
+    if num_sms > max_sms:
+        raise ValueError(f"num_sms ({num_sms}) must not exceed the device SM count ({max_sms})")
+    return num_sms
 
 
 def meta_layout(S: int, K: int, E: int, R: int, NvS: int) -> dict:
@@ -113,10 +145,18 @@ class EmulatedWorld:
     """The communication memory of one emulated EP group on one GPU: every
     rank's ``[NvS, H]`` bf16 shard and meta chunk, side by side.  Buffers
     created with ``world=`` share it, so R Buffers on one GPU see each other's
-    dispatched rows just as R GPUs see each other's symmetric memory."""
+    dispatched rows just as R GPUs see each other's symmetric memory.
+
+    ``host_threads=True`` prepares the world for R host threads, one per rank,
+    each running the reference's per-rank call sequence: ``rendezvous`` is then
+    the emulation of the reference's cross-rank barriers (it blocks the calling
+    thread until all R ranks have arrived and makes every rank's stream wait
+    for the work the other ranks enqueued before arriving).  Without it
+    ``rendezvous`` does nothing.
+    """
 
     def __init__(self, S: int, H: int, K: int, E: int, R: int, token_padding: int = 128,
-                 device=None):
+                 device=None, host_threads: bool = False):
         assert E % R == 0, f"E ({E}) must be divisible by R ({R})"
         epn = E // R
         self.S, self.H, self.K, self.E, self.R, self.token_padding = S, H, K, E, R, token_padding
@@ -124,50 +164,118 @@ class EmulatedWorld:
         self.NvS_padded = self.NvS
         self.layout = meta_layout(S, K, E, R, self.NvS)
         dev = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+        self.device = dev
         self.hidden_buf = torch.empty(R * self.NvS_padded, H, dtype=torch.bfloat16, device=dev)
         self.meta_buf = torch.zeros(R * self.layout["meta_chunk_padded"], dtype=torch.int32,
                                     device=dev)
+        # every rank's dst, deposited by its fresh planning: what the duplicate-group
+        # builder of every destination reads (the reference publishes the same
+        # provenance as src_info in the peers' meta chunks, planning.py:1036-1041)
+        self.dst_all = torch.zeros(R, S * K, dtype=torch.int32, device=dev)
+        self.attached = 0                      # Buffers created on this world
+        self.host_threads = bool(host_threads) and R > 1
+        self._barrier = threading.Barrier(R) if self.host_threads else None
+        self._arrived = [None] * R             # per rank: event recorded on arrival
+        # dup_counts tensors of plans without a duplicate map, by id (a tensor's == is
+        # elementwise, so a WeakSet cannot hold them)
+        self._no_dedup = weakref.WeakValueDictionary()
 
     def matches(self, S, H, K, E, R, token_padding) -> bool:
         return (self.S, self.H, self.K, self.E, self.R, self.token_padding) == \
             (S, H, K, E, R, token_padding)
 
+    # -- gathered tokens_per_expert ------------------------------------------
+    def tpe_table(self, rank: int) -> torch.Tensor:
+        """The ``[R, E]`` count table inside ``rank``'s meta chunk (at TPE_OFF)."""
+        mcp, off = self.layout["meta_chunk_padded"], self.layout["TPE_OFF"]
+        return self.meta_buf[rank * mcp + off: rank * mcp + off + self.R * self.E].view(self.R, self.E)
+
+    def deposit_tokens_per_expert(self, rank: int, row: torch.Tensor) -> None:
+        """Write ``rank``'s ``[E]`` counts into every rank's table, as the
+        reference's planner does into its peers' meta chunks (planning.py:577-583)."""
+        mcp, off = self.layout["meta_chunk_padded"], self.layout["TPE_OFF"] + rank * self.E
+        self.meta_buf.view(self.R, mcp)[:, off: off + self.E].copy_(row.reshape(1, self.E))
+
+    # -- cross-rank barrier ------------------------------------------------------
+    def rendezvous(self, rank: int) -> None:
+        """All R host threads meet here (no-op without ``host_threads``): work that
+        any rank enqueued before arriving is ordered before work that any rank
+        enqueues after leaving, whatever streams the ranks use."""
+        if not self.host_threads:
+            return
+        stream = torch.cuda.current_stream()
+        self._arrived[rank] = stream.record_event()
+        self._barrier.wait()
+        for ev in self._arrived:
+            stream.wait_event(ev)
+        self._barrier.wait()       # nobody re-records before everybody has waited
+
+    def run_ranks(self, fn, *, timeout: float = 120.0):
+        """Run ``fn(rank)`` on R host threads (one per rank) and return the list of
+        results; the first exception of any rank is re-raised.  A rank that fails
+        breaks the barrier so that the others do not wait for it."""
+        assert self.host_threads, "run_ranks needs EmulatedWorld(..., host_threads=True)"
+        results, errors = [None] * self.R, []
+        device = self.device
+
+        def body(r):
+            try:
+                torch.cuda.set_device(device)
+                results[r] = fn(r)
+            except BaseException as exc:  # noqa: BLE001 - reported to the caller below
+                errors.append((r, exc))
+                self._barrier.abort()
+
+        threads = [threading.Thread(target=body, args=(r,), name=f"moonep-rank{r}") for r in range(self.R)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout)
+        alive = [t.name for t in threads if t.is_alive()]
+        if errors:
+            first = [e for e in errors if not isinstance(e[1], threading.BrokenBarrierError)] or errors
+            self._barrier.reset()
+            raise first[0][1]
+        assert not alive, f"rank threads did not finish within {timeout} s: {alive}"
+        return results
+
+    # -- plans without a duplicate map ----------------------------------------------
+    def mark_no_dedup(self, plan: MoonEPCommPlan) -> None:
+        self._no_dedup[id(plan.dup_counts)] = plan.dup_counts
+
+    def has_dedup(self, plan: MoonEPCommPlan) -> bool:
+        return self._no_dedup.get(id(plan.dup_counts)) is not plan.dup_counts
+
 
 def _create_context(S: int, H: int, K: int, E: int, num_ep_ranks: int, num_sms=None,
                     token_padding: int = 128, group=None, rank=None, world=None) -> dict:
-    """Validate the configuration and allocate (or attach to) the buffers.
+    """Validate the configuration, allocate (or attach to) the communication
+    buffers and every scratch buffer a launcher of this context uses.
 
     ``num_sms`` is validated before anything touches the device, as in
-    reference moonep/api.py:231-248.
+    reference moonep/api.py:231-248; shape arithmetic as :260-347.
     """
-    if num_sms is not None:
-        if not isinstance(num_sms, int) or isinstance(num_sms, bool):
-            raise TypeError(f"num_sms must be a positive int, got {type(num_sms).__name__}")
-        if num_sms <= 0:
-            raise ValueError(f"num_sms must be a positive int, got {num_sms}")
-
+    if num_sms is not None and (isinstance(num_sms, bool) or not isinstance(num_sms, int)):
+        raise TypeError(f"num_sms must be a positive int, got {type(num_sms).__name__}")
+    if num_sms is not None and num_sms < 1:
+        raise ValueError(f"num_sms must be a positive int, got {num_sms}")
     device = torch.cuda.current_device()
     max_sms = torch.cuda.get_device_properties(device).multi_processor_count
-    if num_sms is None:
-        num_sms = min(32, max_sms)
-    if num_sms > max_sms:
-        raise ValueError(f"num_sms ({num_sms}) must not exceed the device SM count ({max_sms})")
+    num_sms = _check_num_sms(num_sms, max_sms)
 
     R = num_ep_ranks
     if rank is None:
         import torch.distributed as dist
         rank = dist.get_rank(group=group) if dist.is_available() and dist.is_initialized() else 0
     assert isinstance(rank, int) and 0 <= rank < R, f"rank must be in [0, {R}), got {rank}"
-    N = S * K
     num_sms_dedup = _num_sms_dedup_from_env(max_sms)
 
-    epn = E // R
     assert E % R == 0, f"E ({E}) must be divisible by R ({R})"
     assert isinstance(token_padding, int) and token_padding > 0, \
         f"token_padding must be a positive int, got {token_padding}"
-    NvS_capacity = S * K
+    epn, N = E // R, S * K
     token_padding_extra = (token_padding - 1) * 2 * epn
-    NvS = _align_up(NvS_capacity + token_padding_extra, token_padding)
+    NvS = _align_up(N + token_padding_extra, token_padding)
     int32_max = 2**31 - 1
     assert 0 < N < int32_max, (
         f"planning requires 0 < S*K < int32_max: S={S}, K={K}, S*K={N}, int32_max={int32_max}"
@@ -176,27 +284,26 @@ def _create_context(S: int, H: int, K: int, E: int, num_ep_ranks: int, num_sms=N
         world = EmulatedWorld(S, H, K, E, R, token_padding)
     else:
         assert world.matches(S, H, K, E, R, token_padding), "world was built for another shape"
-    NvS_padded = world.NvS_padded
-    lay = world.layout
+    world.attached += 1
+    NvS_padded, lay = world.NvS_padded, world.layout
     mcp = lay["meta_chunk_padded"]
     max_hidden_index = (R - 1) * NvS_padded + NvS - 1
     assert max_hidden_index <= int32_max, (
         f"dst rank-stride indexing would overflow int32: max_index={max_hidden_index}"
     )
-    hidden_buf, meta_buf = world.hidden_buf, world.meta_buf
-    ctx = {
-        "rank": rank, "group": group, "R": R, "E": E, "S": S, "K": K, "H": H, "N": N,
-        "NvS": NvS, "NvS_capacity": NvS_capacity, "NvS_padded": NvS_padded,
-        "num_sms": num_sms, "num_sms_dedup": num_sms_dedup, "token_padding": token_padding,
-        "device": device, "token_padding_extra": token_padding_extra,
-        "world": world, "hidden_buf": hidden_buf, "meta_buf": meta_buf,
-        "meta_chunk_padded": mcp,
-        **{k: lay[k] for k in ("WEIGHTS_OFF", "TPE_OFF", "PLAN_OFF", "TOPK0_OFF", "ORDER_OFF",
-                               "ORDER0_OFF", "BARRIER_OFF", "SRC_INFO_OFF")},
-        "hidden_buf_local": hidden_buf[rank * NvS_padded: rank * NvS_padded + NvS],
-        "weights_buf_local": meta_buf[rank * mcp + lay["WEIGHTS_OFF"]:
-                                      rank * mcp + lay["WEIGHTS_OFF"] + NvS],
-    }
+    first_row, first_slot = rank * NvS_padded, rank * mcp + lay["WEIGHTS_OFF"]
+    ctx = dict(
+        rank=rank, group=group, R=R, E=E, S=S, K=K, H=H, N=N, NvS=NvS, NvS_capacity=N,
+        NvS_padded=NvS_padded, num_sms=num_sms, num_sms_dedup=num_sms_dedup,
+        token_padding=token_padding, token_padding_extra=token_padding_extra, device=device,
+        world=world, hidden_buf=world.hidden_buf, meta_buf=world.meta_buf, meta_chunk_padded=mcp,
+        hidden_buf_local=world.hidden_buf[first_row: first_row + NvS],
+        weights_buf_local=world.meta_buf[first_slot: first_slot + NvS],
+    )
+    for key in ("WEIGHTS_OFF", "TPE_OFF", "PLAN_OFF", "TOPK0_OFF", "ORDER_OFF", "ORDER0_OFF",
+                "BARRIER_OFF", "SRC_INFO_OFF"):
+        ctx[key] = lay[key]
+    allocate_launch_scratch(ctx)
     if rank == 0:
         logger.info(
             "moonep_amd buffers: R=%d S=%d H=%d E=%d K=%d NvS=%d hidden=%.2f MiB/rank "
@@ -250,33 +357,33 @@ class Buffer:
         return self._ctx
 
     def destroy(self) -> None:
-        """Synchronize and drop every buffer this object holds.  Idempotent."""
-        if self._destroyed:
-            return
-        ctx = self._ctx
-        if ctx is None:
-            self._destroyed = True
-            return
-        if self._comm_stream is not None:
-            self._comm_stream.synchronize()
-        torch.cuda.synchronize()
-        ctx.clear()
+        """Wait for this Buffer's work and let go of every buffer it holds (the
+        world's memory is freed with its last user).  Calling it again is harmless."""
+        if not self._destroyed and self._ctx is not None:
+            if self._comm_stream is not None:
+                self._comm_stream.synchronize()
+            torch.cuda.synchronize()
+            world = self._ctx.get("world")
+            if world is not None:
+                world.attached -= 1
+            self._ctx.clear()
         self._ctx = None
         self._comm_stream = None
         self._destroyed = True
 
     def __del__(self):
+        # a half-constructed object has no _destroyed attribute: nothing to release
         if getattr(self, "_destroyed", True):
             return
         if getattr(self, "explicitly_destroy", False):
             warnings.warn("MoonEP Buffer was not destroyed explicitly; resources may leak.",
                           ResourceWarning)
-            return
-        try:
-            self.destroy()
-        except Exception as exc:  # pragma: no cover - interpreter shutdown
-            warnings.warn(f"MoonEP Buffer destructor failed to destroy resources: {exc!r}",
-                          ResourceWarning)
+        else:
+            try:
+                self.destroy()
+            except Exception as exc:  # pragma: no cover - interpreter shutdown
+                warnings.warn(f"MoonEP Buffer destructor failed to destroy resources: {exc!r}",
+                              ResourceWarning)
 
     # -- helpers -------------------------------------------------------------
     @staticmethod
@@ -303,7 +410,8 @@ class Buffer:
             return comm.record_event()
 
     def _run_dispatch(self, ctx, hidden_sh, route_weights_sk, planning_args, plan, hidden_nvsh,
-                      route_weights_nvs, zero_copy, route_weights_zero_copy) -> None:
+                      route_weights_nvs, zero_copy, route_weights_zero_copy, sync) -> None:
+        world, rank = ctx["world"], int(ctx["rank"])
         dst_all = None
         if planning_args is not None:
             topk, tpe, cu_seqlens = planning_args
@@ -311,30 +419,61 @@ class Buffer:
                 # every rank's routing is known: plan all ranks in one launch
                 # so that this rank's duplicate groups can be built as well
                 dst_all, cu, etc, zfr, stats = launch_planning_all_ranks(ctx, topk, tpe)
-                r = int(ctx["rank"])
-                plan.dst.copy_(dst_all[r])
-                cu_seqlens.copy_(cu[r])
+                plan.dst.copy_(dst_all[rank])
+                cu_seqlens.copy_(cu[rank])
                 plan.experts_to_copy.copy_(etc)
-                plan.zero_fill_ranges.copy_(zfr[r])
-                plan.remote_stats.copy_(stats[r])
+                plan.zero_fill_ranges.copy_(zfr[rank])
+                plan.remote_stats.copy_(stats[rank])
             else:
+                if tpe.dim() == 1 and int(ctx["R"]) > 1:
+                    # the reference's count all-gather: my row into every rank's
+                    # table; the planner reads the table once all rows are in
+                    world.deposit_tokens_per_expert(rank, tpe)
+                    if sync:
+                        world.rendezvous(rank)
+                    tpe = world.tpe_table(rank)
                 launch_planning(ctx, topk.reshape(-1), tpe, cu_seqlens, plan, warm=hidden_sh)
-        launch_dispatch(ctx, hidden_sh, route_weights_sk, plan,
-                        build_dedup_map=planning_args is not None, write_dups=True,
-                        dst_all_ranks=dst_all, pdl_trigger=self.enable_pdl)
+                world.dst_all[rank].copy_(plan.dst)
+        launch_dispatch(ctx, hidden_sh, route_weights_sk, plan, build_dedup_map=False,
+                        write_dups=True, pdl_trigger=self.enable_pdl)
+        if sync:
+            world.rendezvous(rank)   # every rank's rows and dst have landed
+        if planning_args is not None:
+            # duplicate groups are built by the dispatch that follows fresh planning only
+            if dst_all is None and world.host_threads and sync:
+                dst_all = world.dst_all
+            if dst_all is not None:
+                launch_build_dedup(ctx, dst_all, plan)
+            elif int(ctx["R"]) > 1:
+                world.mark_no_dedup(plan)    # the other ranks' dst are not known here
         if not zero_copy:
             hidden_nvsh.copy_(ctx["hidden_buf_local"])
         if route_weights_nvs is not None and not route_weights_zero_copy:
             route_weights_nvs.copy_(ctx["weights_buf_local"].view(torch.float32))
 
     def _run_combine(self, ctx, hidden_sh, plan, hidden_nvsh, route_weights_nvs, route_weights_sk,
-                     zero_copy, router_weights_zero_copy) -> None:
+                     zero_copy, router_weights_zero_copy, sync) -> None:
         if not zero_copy:
             ctx["hidden_buf_local"].copy_(hidden_nvsh)
         if route_weights_nvs is not None and not router_weights_zero_copy:
             ctx["weights_buf_local"].copy_(route_weights_nvs.view(torch.int32))
+        if sync:
+            ctx["world"].rendezvous(int(ctx["rank"]))   # every rank's expert output is in its shard
         launch_combine(ctx, hidden_sh, plan.dst, output_sk=route_weights_sk, mode="two_level",
                        pdl_launch=self.enable_pdl)
+        if sync:
+            ctx["world"].rendezvous(int(ctx["rank"]))   # nobody overwrites a shard that is still read
+
+    def _check_copy_mode(self, ctx, zero_copy: bool, what: str) -> None:
+        """Several Buffers on one world driven from one host thread: a copy taken
+        right after this rank's kernel misses what the other ranks write later."""
+        world = ctx["world"]
+        if not zero_copy and world.attached > 1 and not world.host_threads and int(ctx["R"]) > 1:
+            raise AssertionError(
+                f"{what}(zero_copy=False) on an EmulatedWorld shared by {world.attached} Buffers "
+                "driven from one host thread would copy the shard before the other ranks have "
+                "written (or read) their rows: use zero_copy=True, or a world with "
+                "host_threads=True and one thread per rank")
 
     # -- public operators ------------------------------------------------------
     def dispatch(self, hidden_sh: torch.Tensor, route_weights_sk=None, topk_experts_sk=None,
@@ -344,16 +483,24 @@ class Buffer:
         """Plan (unless ``plan`` is given) and scatter this rank's tokens to
         their expert-grouped slots on every rank.
 
-        Args and return tuple as reference moonep/api.py:713-851.
-        ``tokens_per_expert`` is ``[R, E]``; ``topk_experts_sk`` is ``[S, K]``
-        for this rank, or ``[R, S, K]`` for all ranks -- then the plan also
-        carries this rank's duplicate groups.
+        Args and return tuple as reference moonep/api.py:713-851:
+        ``topk_experts_sk[S, K]`` and ``tokens_per_expert[E]`` of this rank.  The
+        other ranks' counts reach the planner through the world (every rank
+        deposits its row; complete when the ranks run on host threads of a
+        ``host_threads`` world, see the module docstring).  One host thread may
+        pass the gathered ``tokens_per_expert[R, E]`` instead, and
+        ``topk_experts_sk[R, S, K]`` to get this rank's duplicate groups too.
         Returns ``(hidden_nvsh, route_weights_nvs, cu_seqlens, plan[, event])``.
         """
         ctx = self._require_ctx()
+        # the inputs are checked before any kernel (the planner's cache warming
+        # included) reads them
+        check_dispatch_inputs(ctx, hidden_sh, route_weights_sk)
+        self._check_copy_mode(ctx, zero_copy, "dispatch")
         if plan is None:
             assert topk_experts_sk is not None and tokens_per_expert is not None
             assert topk_experts_sk.dtype == torch.int32
+            assert topk_experts_sk.device == hidden_sh.device
             N, R = int(ctx["N"]), int(ctx["R"])
             if topk_experts_sk.dim() == 3:
                 assert topk_experts_sk.numel() == R * N and topk_experts_sk.is_contiguous()
@@ -363,6 +510,7 @@ class Buffer:
             assert tokens_per_expert.dtype == torch.int32
             assert tokens_per_expert.numel() in (int(ctx["E"]), R * int(ctx["E"]))
             assert tokens_per_expert.is_contiguous()
+            assert tokens_per_expert.device == hidden_sh.device
             plan, cu_seqlens = allocate_planning_outputs(ctx)
             planning_args = (topk_experts_sk, tokens_per_expert, cu_seqlens)
         else:
@@ -382,7 +530,8 @@ class Buffer:
 
         def run():
             self._run_dispatch(ctx, hidden_sh, route_weights_sk, planning_args, plan, hidden_nvsh,
-                               route_weights_nvs, zero_copy, router_weights_zero_copy)
+                               route_weights_nvs, zero_copy, router_weights_zero_copy,
+                               bool(inter_rank_sync))
 
         if not async_finish:
             run()
@@ -439,6 +588,7 @@ class Buffer:
         def run():
             launch_prefetch(local_weights, pools, plan.experts_to_copy, scales=scales,
                             rank=int(ctx["rank"]), num_sms=int(ctx["num_sms"]))
+            ctx["world"].rendezvous(int(ctx["rank"]))   # every owner has pushed into every pool
 
         if not async_finish:
             run()
@@ -455,6 +605,7 @@ class Buffer:
         Returns ``(hidden_sh, route_weights_sk | None, event | None)``."""
         ctx = self._require_ctx()
         assert isinstance(plan, MoonEPCommPlan), "Buffer.combine: plan is required"
+        self._check_copy_mode(ctx, zero_copy, "combine")
         assert hidden_nvsh is not None
         assert hidden_nvsh.dtype == torch.bfloat16
         assert hidden_nvsh.is_contiguous()
@@ -483,7 +634,8 @@ class Buffer:
 
         def run():
             self._run_combine(ctx, hidden_sh, plan, hidden_nvsh, route_weights_nvs,
-                              route_weights_sk, zero_copy, router_weights_zero_copy)
+                              route_weights_sk, zero_copy, router_weights_zero_copy,
+                              bool(inter_rank_sync))
 
         if not async_finish:
             run()
@@ -516,9 +668,22 @@ class Buffer:
             assert pool.device == local.device
 
         def run():
+            world, rank = ctx["world"], int(ctx["rank"])
+            if not world.host_threads:
+                for local, pool in zip(local_grads, pools, strict=True):
+                    launch_grad_reduce(local, pool, plan.experts_to_copy, rank=rank,
+                                       num_sms=int(ctx["num_sms"]))
+                return
+            # ranks on host threads: every rank reads before any rank clears, as the
+            # reference's barrier between the two halves ensures (grad_reduce.py:369-372)
+            world.rendezvous(rank)
             for local, pool in zip(local_grads, pools, strict=True):
-                launch_grad_reduce(local, pool, plan.experts_to_copy, rank=int(ctx["rank"]),
-                                   num_sms=int(ctx["num_sms"]))
+                launch_grad_reduce(local, pool, plan.experts_to_copy, rank=rank,
+                                   num_sms=int(ctx["num_sms"]), phase="reduce")
+            world.rendezvous(rank)
+            for local, pool in zip(local_grads, pools, strict=True):
+                launch_grad_reduce(local, pool, plan.experts_to_copy, rank=rank,
+                                   num_sms=int(ctx["num_sms"]), phase="clear")
 
         if not async_finish:
             run()

@@ -24,6 +24,8 @@ def launch_combine_prologue(ctx: dict, plan: MoonEPCommPlan, *, pdl_trigger: boo
     """In place on the local shard: primary row <- bf16(fp32 sum of the
     primary and its duplicate rows)."""
     assert isinstance(plan, MoonEPCommPlan)
+    from .dispatch import _require_dedup_map
+    _require_dedup_map(ctx, plan, "launch_combine_prologue")
     H, NvS = int(ctx["H"]), int(ctx["NvS"])
     shard = ctx["hidden_buf_local"]
     assert shard.dtype == torch.bfloat16 and shard.is_contiguous()

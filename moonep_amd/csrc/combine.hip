@@ -159,7 +159,12 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(CombineArgs a) {
       mep_u4 o;
 #pragma unroll
       for (int j = 0; j < 4; ++j) o[j] = mep_pack_bf16(acc[i][2 * j], acc[i][2 * j + 1]);
-      mep_st16_stream(orow + (size_t)i * 1024, o);
+      // Store policy measured per mode at S=4096, H=7168 (same machine, runs
+      // alternated): the one-wave-per-token modes gain 1.2-1.4 us of 87 with
+      // stores written through at system scope, the two-level mode loses 4 us
+      // of 88 with them (also with 7-chunk tiles) and keeps the nontemporal hint.
+      if (TWO) mep_st16_stream(orow + (size_t)i * 1024, o);
+      else mep_st16_through(orow + (size_t)i * 1024, o);
     }
   }
 }

@@ -318,7 +318,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   int e = -1;
   if (tid < n) {
     e = topk[e0 + tid];
-    if ((unsigned)e >= (unsigned)E) e = -1;  // invalid id: slot 0, never out of bounds
+    if ((unsigned)e >= (unsigned)E) e = -1;  // invalid id: becomes an entry that nobody copies
   }
   // lanes of my wave holding the same expert: one ballot per key bit
   int pos = 0;
@@ -337,8 +337,12 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
     }
   }
   __syncthreads();
-  int dv = 0, dest = 0;
+  // An entry with an invalid expert id gets destination rank R: dispatch and
+  // combine skip such entries (they never write or read outside the R shards),
+  // the duplicate-group builder matches no rank to it.
+  int dv = (int)min((int64_t)R * NvS, (int64_t)INT32_MAX), dest = -1;
   if (e >= 0) {
+    dest = 0;
     int before = 0;
     for (int w4 = 0; w4 <= (wave >> 2); ++w4) {
       const unsigned word = (unsigned)s_wcnt[e * W4 + w4];
@@ -375,7 +379,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   if (tid < n) {
     const int k = tid % K;
     bool dup = false;
-    for (int j = tid - k; j < tid; ++j) dup |= (s_cd[j] == dest);
+    for (int j = tid - k; j < tid; ++j) dup |= (dest >= 0 && s_cd[j] == dest);
     dst[e0 + tid] = dup ? -dv - 1 : dv;
   }
 }
@@ -399,6 +403,20 @@ struct PlanConfig {
   int tok_per_wg;
   int groups;
 };
+
+// CUs of the current device, asked once per device
+int device_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return -1;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
 
 // 0 on success
 int plan_config(int S, int K, int E, int R, PlanConfig* c) {
@@ -468,7 +486,12 @@ int plan_launch(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int n
   if (a.warm_vecs) {
     const size_t per_wg = (size_t)c.nt * 8;
     const size_t want = (a.warm_vecs + per_wg - 1) / per_wg;
-    const size_t cap = c.nt == 1024 ? 480 : 1920;
+    // what the CUs hold beside the planning workgroups at 2048 threads per CU
+    // (480 workgroups of 1024 threads on 256 CUs)
+    const int cus = device_cu_count();
+    if (cus <= 0) return MEP_ERR_INVALID_ARG;
+    const int64_t room = (int64_t)cus * (2048 / c.nt) - (int64_t)c.groups * nranks;
+    const size_t cap = room > 0 ? (size_t)room : 0;
     warm_groups = (int)(want < cap ? want : cap);
   }
   dim3 grid(c.groups + warm_groups, nranks);

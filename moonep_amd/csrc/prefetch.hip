@@ -180,6 +180,7 @@ struct ReduceArgs {
   int64_t elems;        // per expert
   const int* etc;
   int rank, epn, R;
+  unsigned flags;       // MEP_REDUCE_*
 };
 
 typedef float mep_f4 __attribute__((ext_vector_type(4)));
@@ -215,7 +216,9 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
     for (int c = 0; c < a.epn; c += 64) {
       const int b = c + lane;
       const int e = b < a.epn ? a.etc[a.rank * a.epn + b] : -1;
-      const bool foreign = e >= 0 && (unsigned)(e - lo) >= (unsigned)a.epn;
+      // a clear-only call zeroes every occupied own slot as tiles
+      const bool foreign = e >= 0 && ((a.flags & MEP_REDUCE_CLEAR_ONLY) ||
+                                      (unsigned)(e - lo) >= (unsigned)a.epn);
       const uint64_t m = __ballot(foreign);
       if (foreign) occ[n + __popcll(m & mep_lanes_lt())] = b;
       n += __popcll(m);
@@ -223,8 +226,9 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
     if (lane == 0) occ[a.epn] = n;
   }
   t.build(a.etc, a.rank, a.R, a.epn);  // ends with a workgroup barrier
-  const int n_active = t.misc[0];
-  const int n_clear = occ[a.epn];
+  const int n_active = (a.flags & MEP_REDUCE_CLEAR_ONLY) ? 0 : t.misc[0];
+  const int n_clear = (a.flags & MEP_REDUCE_NO_CLEAR) ? 0 : occ[a.epn];
+  const bool clear_as_read = a.flags == 0;  // own slots holding own experts, zeroed by their reader
   if (n_active == 0 && n_clear == 0) return;
   const int64_t vecs = a.elems / 4;
   constexpr int kTileVecs = kBlock * kVecPerThread;
@@ -252,7 +256,7 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
     // slot sidx belongs to `rank` itself (it then holds one of the rank's own experts)
     auto own_slot = [&](int sidx) -> int {
       const int rb = t.list[sidx];
-      return rb / a.epn == a.rank ? rb - a.rank * a.epn : -1;
+      return (clear_as_read && rb / a.epn == a.rank) ? rb - a.rank * a.epn : -1;
     };
     mep_f4 acc[kVecPerThread];
     if ((tile + 1) * kTileVecs <= vecs) {
@@ -353,7 +357,8 @@ extern "C" int mep_prefetch(int ntensors, const void* const* local, void* const*
 
 extern "C" int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t rank_stride_elems,
                                const int32_t* experts_to_copy, int rank, int epn, int R,
-                               int64_t elems_per_expert, void* stream) {
+                               int64_t elems_per_expert, unsigned flags, void* stream) {
+  MEP_REQUIRE(flags <= MEP_REDUCE_CLEAR_ONLY, MEP_ERR_INVALID_ARG);  // the two flags exclude each other
   MEP_REQUIRE(local_grad && reduce_pool && experts_to_copy, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(epn > 0 && R > 0 && rank >= 0 && rank < R && elems_per_expert > 0,
               MEP_ERR_INVALID_ARG);
@@ -364,7 +369,7 @@ extern "C" int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t ra
   const size_t lds = slot_table_bytes(R, epn) + ((size_t)epn + 1) * sizeof(int);  // + own foreign-held slots
   MEP_REQUIRE(lds <= 64 * 1024, MEP_ERR_UNSUPPORTED);
   ReduceArgs a{local_grad, reduce_pool, rank_stride_elems, elems_per_expert, experts_to_copy,
-               rank, epn, R};
+               rank, epn, R, flags};
   const int64_t tiles = (elems_per_expert / 4 + kBlock * kVecPerThread - 1) /
                         (kBlock * kVecPerThread);
   const int blocks = stream_blocks(tiles, R, epn, 512);

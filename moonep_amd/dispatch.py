@@ -34,6 +34,33 @@ def _check_dispatch_plan(ctx: dict, hidden_sh: torch.Tensor, plan: MoonEPCommPla
     chk(plan.dup_counts, "dup_counts", (2,))
 
 
+def check_dispatch_inputs(ctx: dict, hidden_sh, route_weights_sk) -> None:
+    """The token and weight tensors of a dispatch, checked as reference
+    moonep/dispatch.py:880-905 checks them (no device access)."""
+    H, S, K = (int(ctx[k]) for k in ("H", "S", "K"))
+    assert hidden_sh.dtype == torch.bfloat16 and hidden_sh.is_contiguous(), \
+        "hidden_sh must be contiguous bf16"
+    assert hidden_sh.is_cuda, "hidden_sh must be a CUDA tensor"
+    assert tuple(hidden_sh.shape) == (S, H), \
+        f"hidden_sh must be shape [S={S}, H={H}], got {tuple(hidden_sh.shape)}"
+    assert ctx["hidden_buf"].device == hidden_sh.device
+    if route_weights_sk is not None:
+        assert route_weights_sk.dtype == torch.float32 and route_weights_sk.is_contiguous(), \
+            "route_weights_sk must be contiguous fp32"
+        assert tuple(route_weights_sk.shape) == (S, K), \
+            f"route_weights_sk must be shape [S={S}, K={K}], got {tuple(route_weights_sk.shape)}"
+        assert route_weights_sk.device == hidden_sh.device
+    assert H % 8 == 0, "H must be multiple of 8 for 16-B row vectors"
+
+
+def _require_dedup_map(ctx: dict, plan: MoonEPCommPlan, what: str) -> None:
+    world = ctx.get("world")
+    assert world is None or world.has_dedup(plan), (
+        f"{what}: this plan has no duplicate map (it was planned from one rank's topk only, so "
+        "the other ranks' dst were unknown); plan with topk[R, S, K], or drive the ranks from "
+        "host threads of an EmulatedWorld(host_threads=True)")
+
+
 def launch_dispatch(ctx: dict, hidden_sh, route_weights_sk, plan, *, build_dedup_map: bool = True,
                     pdl_trigger: bool = False, write_dups: bool = False,
                     dst_all_ranks: torch.Tensor | None = None) -> None:
@@ -49,20 +76,8 @@ def launch_dispatch(ctx: dict, hidden_sh, route_weights_sk, plan, *, build_dedup
     """
     assert isinstance(plan, MoonEPCommPlan)
     H, R, S, K, E = (int(ctx[k]) for k in ("H", "R", "S", "K", "E"))
-    assert hidden_sh.dtype == torch.bfloat16 and hidden_sh.is_contiguous(), \
-        "hidden_sh must be contiguous bf16"
-    assert hidden_sh.is_cuda, "hidden_sh must be a CUDA tensor"
-    assert tuple(hidden_sh.shape) == (S, H), \
-        f"hidden_sh must be shape [S={S}, H={H}], got {tuple(hidden_sh.shape)}"
+    check_dispatch_inputs(ctx, hidden_sh, route_weights_sk)
     _check_dispatch_plan(ctx, hidden_sh, plan)
-    assert ctx["hidden_buf"].device == hidden_sh.device
-    if route_weights_sk is not None:
-        assert route_weights_sk.dtype == torch.float32 and route_weights_sk.is_contiguous(), \
-            "route_weights_sk must be contiguous fp32"
-        assert tuple(route_weights_sk.shape) == (S, K), \
-            f"route_weights_sk must be shape [S={S}, K={K}], got {tuple(route_weights_sk.shape)}"
-        assert route_weights_sk.device == hidden_sh.device
-    assert H % 8 == 0, "H must be multiple of 8 for 16-B row vectors"
     meta = ctx["meta_buf"]
     wslots = None
     if route_weights_sk is not None:
@@ -100,6 +115,7 @@ def launch_build_dedup(ctx: dict, dst_all_ranks: torch.Tensor, plan: MoonEPCommP
 def launch_dispatch_epilogue(ctx: dict, plan: MoonEPCommPlan, *, pdl_launch: bool = False) -> None:
     """Copy every primary row of the local shard to its duplicate rows."""
     assert isinstance(plan, MoonEPCommPlan)
+    _require_dedup_map(ctx, plan, "launch_dispatch_epilogue")
     shard = ctx["hidden_buf_local"]
     assert shard.dtype == torch.bfloat16 and shard.is_contiguous()
     rc = _lib.lib().mep_dispatch_epilogue(

@@ -20,7 +20,8 @@ import torch
 from . import _lib
 
 
-def launch_grouped_gemm_nt(rows, weights, cu_seqlens, out=None, *, up_weights=None, row_scale=None):
+def launch_grouped_gemm_nt(rows, weights, cu_seqlens, out=None, *, up_weights=None, row_scale=None,
+                           token_padding: int = 128):
     """``out[m] = rows[m] @ weights[g(m)].T`` (fp32 accumulation, bf16 out).
 
     rows [M,K] bf16; weights [G,N,K] bf16; cu_seqlens [G] int32 on the device,
@@ -28,8 +29,13 @@ def launch_grouped_gemm_nt(rows, weights, cu_seqlens, out=None, *, up_weights=No
     ``silu(rows @ weights[g].T) * (rows @ up_weights[g].T)``; otherwise
     ``row_scale`` [M] fp32 (optional) multiplies each row.  Rows at or beyond
     ``cu_seqlens[-1]`` are not written (``out`` is zero-filled when allocated
-    here).
+    here).  ``token_padding`` is the padding the plan behind ``cu_seqlens`` was
+    made with: the kernel gives every 128-row tile to ONE group, so group ends
+    must be multiples of 128 (checked here on the host, no device read).
     """
+    assert isinstance(token_padding, int) and token_padding > 0 and token_padding % 128 == 0, (
+        f"grouped GEMM needs group ends on 128-row tiles: token_padding must be a multiple of "
+        f"128, got {token_padding}")
     assert rows.is_cuda and rows.dtype == torch.bfloat16 and rows.is_contiguous() and rows.dim() == 2
     assert weights.dtype == torch.bfloat16 and weights.is_contiguous() and weights.dim() == 3
     M, K = rows.shape
@@ -53,9 +59,12 @@ def launch_grouped_gemm_nt(rows, weights, cu_seqlens, out=None, *, up_weights=No
     return out
 
 
-def grouped_ffn_hip(rows, slots, cu_seqlens, gate_t, up_t, down):
+def grouped_ffn_hip(rows, slots, cu_seqlens, gate_t, up_t, down, *, token_padding: int = 128):
     """SwiGLU FFN of one rank's rows.  rows [NvS,H] bf16, slots [NvS] fp32 route
     weights (or None), cu_seqlens [2*epn]; gate_t/up_t [2*epn,H',H], down
-    [2*epn,H,H'].  Rows outside every group come out as zeros."""
-    hmid = launch_grouped_gemm_nt(rows, gate_t, cu_seqlens, up_weights=up_t)
-    return launch_grouped_gemm_nt(hmid, down, cu_seqlens, row_scale=slots)
+    [2*epn,H,H'].  Rows outside every group come out as zeros.  ``token_padding``:
+    that of the Buffer whose plan produced ``cu_seqlens`` (a multiple of 128)."""
+    hmid = launch_grouped_gemm_nt(rows, gate_t, cu_seqlens, up_weights=up_t,
+                                  token_padding=token_padding)
+    return launch_grouped_gemm_nt(hmid, down, cu_seqlens, row_scale=slots,
+                                  token_padding=token_padding)

@@ -13,14 +13,19 @@ N_BLOCK = 128
 
 def launch_grad_reduce(local_expert_grads, reduce_buffers, experts_to_copy, rank, num_sms=None,
                        meta_buf=None, meta_stride=None, barrier_off=None,
-                       grid_sync_bar=None) -> None:
+                       grid_sync_bar=None, *, phase: str = "both") -> None:
     """``local_expert_grads[le] += sum of reduce_buffers[src, b]`` over the
     slots holding expert ``rank*epn+le`` in (src, b)-ascending order, then zero
     ``reduce_buffers[rank, b]`` for every occupied slot b of this rank.
 
+    ``phase`` (not in the reference): "both" (one launch), "reduce" (sum only)
+    or "clear" (zero the own occupied slots only).  The reference puts a
+    cross-rank barrier between the two halves; whoever drives several ranks on
+    one GPU calls "reduce" for every rank, then "clear" for every rank.
     ``num_sms`` and the barrier arguments of the reference are accepted and
     unused.
     """
+    flags = {"both": 0, "reduce": _lib.REDUCE_NO_CLEAR, "clear": _lib.REDUCE_CLEAR_ONLY}[phase]
     if reduce_buffers.numel() == 0 or experts_to_copy.numel() == 0:
         return
     assert local_expert_grads.dtype == torch.float32 and local_expert_grads.is_contiguous(), \
@@ -52,6 +57,6 @@ def launch_grad_reduce(local_expert_grads, reduce_buffers, experts_to_copy, rank
     assert reduce_buffers.device == dev and experts_to_copy.device == dev
     rc = _lib.lib().mep_grad_reduce(
         local_expert_grads.data_ptr(), reduce_buffers.data_ptr(), int(reduce_buffers.stride(0)),
-        experts_to_copy.data_ptr(), int(rank), epn, R, H * Hp, _lib.current_stream(),
+        experts_to_copy.data_ptr(), int(rank), epn, R, H * Hp, flags, _lib.current_stream(),
     )
     _lib.check(rc, "mep_grad_reduce")

@@ -137,9 +137,9 @@ class _GroupPrefetch(torch.autograd.Function):
         grad = g_views[:, :epn].float().contiguous()
         slots = g_views[:, epn:].float().contiguous()
         for r in range(R):
-            # every rank reads before any rank clears (a barrier in the reference):
-            # each emulated rank works on its own copy of the slot grads
-            launch_grad_reduce(grad[r], slots.clone(), ctx.etc, rank=r)
+            # every rank reads before any rank clears (a barrier in the reference): only
+            # the summing half runs here, the slot grads are temporaries nobody reads again
+            launch_grad_reduce(grad[r], slots, ctx.etc, rank=r, phase="reduce")
         return None, None, grad
 
 

@@ -119,6 +119,11 @@ def _check_dedup_encoding_bounds(ctx: dict) -> None:
 
 
 def _tpe_table(ctx: dict, tokens_per_expert: torch.Tensor) -> torch.Tensor:
+    """The ``[R, E]`` count table the planner reads.  A per-rank ``[E]`` row is
+    deposited into the world's gathered table (the reference's planner writes
+    its row into its peers' meta chunks, planning.py:577-583) and the table of
+    this rank's meta chunk is returned; the caller has to make sure the other
+    ranks' rows are in (``EmulatedWorld.rendezvous``) before the launch."""
     R, E = int(ctx["R"]), int(ctx["E"])
     assert tokens_per_expert.dtype == torch.int32 and tokens_per_expert.is_contiguous()
     if tokens_per_expert.dim() == 2:
@@ -129,21 +134,32 @@ def _tpe_table(ctx: dict, tokens_per_expert: torch.Tensor) -> torch.Tensor:
     assert tokens_per_expert.numel() == E
     if R == 1:
         return tokens_per_expert.reshape(1, E)
-    raise NotImplementedError(
-        "one GPU stands in for all R ranks here: pass every rank's counts as "
-        "tokens_per_expert[R, E] (the reference gathers them from peer GPUs)"
-    )
+    world, rank = ctx["world"], int(ctx["rank"])
+    world.deposit_tokens_per_expert(rank, tokens_per_expert)
+    return world.tpe_table(rank)
 
 
 def plan_scratch(ctx: dict, nranks: int = 1) -> torch.Tensor | None:
     """Device scratch the planner needs for this shape (None when its tables
-    fit in LDS); cached in ctx."""
+    fit in LDS).  ``allocate_launch_scratch`` fills the cache for one rank and
+    for all R ranks when the context is made, so no launcher allocates."""
     key = ("plan_scratch", nranks)
     if key not in ctx:
         n = _lib.lib().mep_plan_scratch_bytes(ctx["S"], ctx["K"], ctx["E"], ctx["R"], nranks)
         ctx[key] = (torch.empty(n, dtype=torch.uint8, device=ctx["meta_buf"].device)
                     if n else None)
     return ctx[key]
+
+
+def allocate_launch_scratch(ctx: dict) -> None:
+    """Every scratch buffer the launchers of this context use, allocated once:
+    the planner's tables (one rank / all ranks) and the duplicate-group
+    builder's counters."""
+    lib = _lib.lib()
+    plan_scratch(ctx, 1)
+    plan_scratch(ctx, int(ctx["R"]))
+    n = lib.mep_dedup_scratch_bytes(int(ctx["S"]), int(ctx["R"]))
+    ctx["dedup_scratch"] = torch.empty(n, dtype=torch.uint8, device=ctx["meta_buf"].device)
 
 
 def launch_planning(ctx: dict, topk_experts_flat, tokens_per_expert, cu_seqlens, plan, *,

@@ -182,7 +182,7 @@ int main() {
   HIP_OK(d_grad.alloc(grad.size())); HIP_OK(d_grad.up(grad));
   HIP_OK(d_red.alloc(red.size())); HIP_OK(d_red.up(red));
   ora_grad_reduce(grad.data(), red.data(), epn * elems, elems, etc_ref.data(), rank, epn, R);
-  MEP_OK_(mep_grad_reduce(d_grad.p, d_red.p, epn * elems, d_etc.p, rank, epn, R, elems, nullptr));
+  MEP_OK_(mep_grad_reduce(d_grad.p, d_red.p, epn * elems, d_etc.p, rank, epn, R, elems, 0u, nullptr));
   HIP_OK(hipDeviceSynchronize());
   HIP_OK(d_grad.down(got_f)); bad += same("grad reduce local grads", got_f, grad);
   HIP_OK(d_red.down(got_f)); bad += same("grad reduce pool after clears", got_f, red);

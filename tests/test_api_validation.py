@@ -142,3 +142,15 @@ def test_routing_generators():
     topk2, *_ = routing.logit_routing(256, 8, 64, 8, 1.0, seed=3)
     assert torch.equal(topk, topk2)
     assert routing.pattern("duplicate_topk", 4, 3, 8, 4, 1).unique().tolist() == [4]
+
+
+def test_grouped_gemm_rejects_paddings_that_split_a_tile():
+    """The grouped GEMM gives every 128-row tile to one group: a plan made with a
+    smaller token_padding is refused on the host, before any tensor is looked at."""
+    from moonep_amd.ffn import grouped_ffn_hip, launch_grouped_gemm_nt
+    x = torch.zeros(128, 64, dtype=torch.bfloat16)
+    for tp in (16, 64, 192, 0):
+        with pytest.raises(AssertionError, match="multiple of 128"):
+            launch_grouped_gemm_nt(x, x, x, token_padding=tp)
+        with pytest.raises(AssertionError, match="multiple of 128"):
+            grouped_ffn_hip(x, None, x, x, x, x, token_padding=tp)

@@ -41,7 +41,7 @@ def test_argument_validation_needs_no_device():
     assert lib.mep_plan(None, None, 0, 4, 2, 8, 2, 8, 64, None, None, None, None, None, None, 0, None) == -1
     assert lib.mep_dispatch(None, None, None, None, None, 0, None, 0, 0, 4, 64, 2, 2, 4, 64, 8, 0, None) == -1
     assert lib.mep_combine(None, 0, None, 0, None, None, None, 4, 64, 2, 2, 64, 0, None) == -1
-    assert lib.mep_grad_reduce(None, None, 0, None, 0, 4, 2, 16, None) == -1
+    assert lib.mep_grad_reduce(None, None, 0, None, 0, 4, 2, 16, 0, None) == -1
     assert lib.mep_plan_scratch_bytes(4096, 8, 256, 8, 1) == 0          # tables fit in LDS
     assert lib.mep_plan_scratch_bytes(256, 1, 2050, 2, 2) > 0           # they do not
     assert lib.mep_dedup_scratch_bytes(4096, 8) >= 4096 * 8 * 4
@@ -88,9 +88,10 @@ def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
     assert lib.mep_combine(A, 64, None, 0, A, A, None, 4, 60, 2, 2, 64, 0, None) == -2     # H % 8 != 0
     assert lib.mep_combine(A, 64, None, 0, A, A, None, 4, 64, 33, 2, 64, 0, None) == -2    # K > 32
     assert lib.mep_combine(A, 32, None, 0, A, A, None, 4, 64, 2, 2, 64, 0, None) == -1     # stride < NvS
-    assert lib.mep_grad_reduce(A, A, 16 * 4, A, 0, 4, 2, 18, None) == -2                   # elems % 4 != 0
-    assert lib.mep_grad_reduce(A, A, 8, A, 0, 4, 2, 16, None) == -1                        # stride too small
-    assert lib.mep_grad_reduce(A + 4, A, 64, A, 0, 4, 2, 16, None) == -4
+    assert lib.mep_grad_reduce(A, A, 16 * 4, A, 0, 4, 2, 18, 0, None) == -2                   # elems % 4 != 0
+    assert lib.mep_grad_reduce(A, A, 8, A, 0, 4, 2, 16, 0, None) == -1                      # stride too small
+    assert lib.mep_grad_reduce(A + 4, A, 64, A, 0, 4, 2, 16, 0, None) == -4
+    assert lib.mep_grad_reduce(A, A, 64, A, 0, 4, 2, 16, 3, None) == -1                        # both phase flags at once
     # grouped GEMM: tile multiples, swiglu needs the up weights and no row scale
     assert lib.mep_grouped_gemm_nt(A, A, None, A, 4, A, None, 100, 256, 64, 0, None) == -2
     assert lib.mep_grouped_gemm_nt(A, A, None, A, 4, A, None, 128, 128, 64, 0, None) == -2

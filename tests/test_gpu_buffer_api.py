@@ -155,8 +155,11 @@ def test_bad_inputs_raise_like_the_reference(cuda):
         b.dispatch(hid_d, w_d)                                   # neither plan nor routing
     with pytest.raises(AssertionError):
         b.dispatch(hid_d, w_d, topk_d.long(), tpe_d)             # wrong dtype
-    with pytest.raises(NotImplementedError, match=r"tokens_per_expert\[R, E\]"):
-        b.dispatch(hid_d, w_d, topk_d, tpe_d[0].contiguous())    # one rank's counts only
+    # one rank's counts only: the reference's call shape.  The row goes into the world's
+    # gathered table; with nobody playing the other ranks their rows stay zero
+    _, _, _, lone = b.dispatch(hid_d, w_d, topk_d, tpe_d[0].contiguous())
+    assert isinstance(lone, MoonEPCommPlan)
+    assert torch.equal(b._require_ctx()["world"].tpe_table(0)[0], tpe_d[0])
     with pytest.raises(AssertionError, match="hidden_sh"):
         b.dispatch(hid_d.float(), w_d, topk_d, tpe_d)
     with pytest.raises(AssertionError, match="hidden_sh"):

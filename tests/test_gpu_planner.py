@@ -203,3 +203,56 @@ def test_planner_with_cache_warming_is_the_same_planner(cuda, S, K, E, R, tp, wa
     assert np.array_equal(plan.remote_stats.cpu().numpy(), plans[rank].remote_stats)
     assert torch.equal(warm.view(torch.int16), before.view(torch.int16))
     buf.destroy()
+
+
+def test_invalid_expert_ids_become_entries_that_nobody_copies(cuda):
+    """An id outside [0, E) gets destination rank R (dst = R*NvS, never marked a
+    duplicate): dispatch writes nothing for it, combine reads nothing, the other
+    entries are planned as if it were not there."""
+    from moonep_amd.combine import launch_combine
+    from moonep_amd.dispatch import launch_dispatch
+    from oracle import ops_oracle as oo
+    S, H, K, E, R, tp, rank = 96, 256, 4, 12, 3, 8, 1
+    topk = torch.stack([routing.popularity_biased(S, K, E, R, r, 1.0, seed=9) for r in range(R)])
+    bad = topk[rank].clone()
+    bad[3, 1] = E            # one past the last expert
+    bad[3, 2] = -5           # negative
+    bad[40, 0] = 1 << 20
+    bad[95, 3] = E + 7
+    valid = (bad >= 0) & (bad < E)
+    tpe = routing.tokens_per_expert(topk, E)
+    flat = bad.reshape(-1)
+    tpe[rank] = torch.bincount(flat[valid.reshape(-1)].long(), minlength=E).to(torch.int32)
+    gp = po.plan_global(tpe.numpy(), S, K, tp)
+    NvS = gp.NvS
+    raw = np.full(S * K, R * NvS, dtype=np.int64)
+    vmask = valid.reshape(-1).numpy()
+    raw[vmask] = po.raw_dst_for_rank(gp, flat.numpy()[vmask], rank)
+    want = po.canonicalize_dst(raw, K, NvS)
+    want[~vmask] = R * NvS                      # an invalid entry is never a duplicate
+    buf = Buffer(S, H, K, E, R, token_padding=tp, rank=rank)
+    ctx = buf._require_ctx()
+    ctx["hidden_buf"].fill_(-3.0)
+    plan, cu = allocate_planning_outputs(ctx)
+    launch_planning(ctx, flat.contiguous().to(cuda), tpe.to(cuda), cu, plan)
+    torch.cuda.synchronize()
+    assert np.array_equal(plan.dst.cpu().numpy(), want.astype(np.int32))
+    assert np.array_equal(cu.cpu().numpy(), gp.cu_seqlens[rank])
+    # rows: only the valid entries are written, nothing outside the shards is touched
+    g = torch.Generator().manual_seed(2)
+    hid = torch.randint(-4, 5, (S, H), generator=g).to(torch.bfloat16)     # small integers: exact sums
+    launch_dispatch(ctx, hid.to(cuda), None, plan, build_dedup_map=False, write_dups=True)
+    out = torch.empty(S, H, dtype=torch.bfloat16, device=cuda)
+    launch_combine(ctx, out, plan.dst, mode="all")
+    torch.cuda.synchronize()
+    shards = ctx["hidden_buf"].view(R, NvS, H).cpu()
+    written = torch.zeros(R * NvS, dtype=torch.bool)
+    written[torch.from_numpy(raw[vmask])] = True
+    for d in range(R):
+        zf = gp.zero_fill[d] if d == rank else None
+        if zf is not None:
+            for start, n in zf:
+                written[d * NvS + int(start): d * NvS + int(start) + int(n)] = True
+    assert bool((shards.view(R * NvS, H)[~written] == -3.0).all())
+    assert torch.equal(out.cpu().float(), hid.float() * valid.sum(1, keepdim=True).float())
+    buf.destroy()
