@@ -2,16 +2,24 @@
 MI355X at S=4096, H=7168, K=8, E=256, R=8, token_padding=128, bf16, routing at
 maxvio ~= 1 (synthetic, seeded).
 
-    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--full]
+    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--chain-only]
 
 A step is one pass planner -> dispatch -> combine over one of six rotating
 token sets; the K timed steps are recorded into one HIP graph and replayed
-once (K single-step replays are timed beside it).  Prints ONE JSON line.  `value` is the chain's throughput:
-algorithmic bytes of dispatch + combine (each S*H*2 + S*K*H*2) divided by the
-time of a whole step (planner included), in GB/s, inputs resident in HBM.
-Per-kernel durations are measured with HIP events on the launching stream;
-the dominant kernel's figure feeds `roofline`.  `--full` adds the maxvio
-sweep, the second shape, prefetch_weight and reduce_grad to the JSON line.
+once (K single-step replays are timed beside it).  Prints ONE JSON line.
+`value` is the chain's throughput: algorithmic bytes of dispatch + combine
+(each S*H*2 + S*K*H*2) divided by the time of a whole step (planner included),
+in GB/s, inputs resident in HBM.  Per-kernel durations are measured with HIP
+events on the launching stream.  `roofline` describes the dominant kernel from
+its COLD, standalone duration (every launch reads a token set that is not in
+any cache); its duration inside the timed steps, where the planner launch has
+already pulled the tokens into the last-level cache, is reported beside it.
+
+The same line carries the other configurations: the chain at maxvio 0 .. 4 on
+both shapes (`maxvio_sweep`), prefetch_weight and reduce_grad at
+[32, 7168, 2048] per rank for the planner's own slot table and for a table with
+8 slots per rank (`weights`), and the expert-side grouped FFN (`ffn`), each
+with its own `roofline` record.  `--chain-only` skips them.
 
 The CPU baseline is the scalar C restatement of the same chain
 (oracle/mep_oracle.c), timed on the host next to the GPU.
@@ -20,17 +28,45 @@ The CPU baseline is the scalar C restatement of the same chain
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
 import sys
 import time
 
 HBM_PEAK_GBPS = 8000.0
+ROOT = os.path.dirname(os.path.abspath(__file__))
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
-# HBM-side bytes per launch (L2 fetches + writes) from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs, scaled by the factors a 512 MiB copy gives (2.000 and 1.000);
-# the summary is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"dispatch": 119.7e6 + 498.4e6, "combine": 472.0e6 + 58.9e6}
+
+def kernel_source_digest() -> str:
+    """Identifies the kernel sources a traffic measurement belongs to."""
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "moonep_amd", "csrc")
+    for name in ("mep_common.h", "dispatch.hip", "combine.hip"):
+        with open(os.path.join(csrc, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(kernel: str, grid: int):
+    """(HBM-side bytes per launch, note) for `kernel` from profiles/traffic.json: L2
+    fetches + writes counted by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by the
+    factors a 512 MiB copy gives.  The figure is only used when the file was made from the
+    kernel sources and the launch grid that run now; otherwise (None, why)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError) as exc:
+        return None, f"no traffic record: {exc}"
+    if rec.get("source_digest") != kernel_source_digest():
+        return None, "profiles/traffic.json was measured on other kernel sources: re-run the PMC profile"
+    k = rec.get("kernels", {}).get(kernel)
+    if k is None:
+        return None, f"profiles/traffic.json has no entry for {kernel}"
+    if int(k.get("grid", -1)) != int(grid):
+        return None, f"profiles/traffic.json: {kernel} was measured with grid {k.get('grid')}, not {grid}"
+    return float(k["fetch_bytes"]) + float(k["write_bytes"]), None
 
 
 def parse():
@@ -38,7 +74,12 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--full", action="store_true", help="also sweep maxvio, 2nd shape, prefetch, grad reduce")
+    ap.add_argument("--chain-only", action="store_true",
+                    help="config 1 only: skip the maxvio sweep, prefetch / grad reduce and the FFN")
+    ap.add_argument("--full", action="store_true", help="accepted for older command lines; everything runs by default")
+    ap.add_argument("--write-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: turn the counter_collection.csv files of two rocprofv3 --pmc runs of "
+                         "`bench.py --profile-kernels` (FETCH_SIZE, WRITE_SIZE) into profiles/traffic.json")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--profile-kernels", action="store_true",
                     help="for rocprofv3: a few plain launches of each kernel and of a 512 MiB "
@@ -46,6 +87,15 @@ def parse():
     ap.add_argument("--maxvio", type=float, default=1.0)
     ap.add_argument("--seed", type=int, default=2024)
     return ap.parse_args()
+
+
+def hbm_roofline(kernel, algorithmic_bytes, us, traffic=None, **extra):
+    """A roofline record of an HBM-bound kernel: algorithmic bytes per launch over its
+    average launch duration against the 8 TB/s of MI355X."""
+    achieved = algorithmic_bytes / us / 1e3 if us > 0 and algorithmic_bytes else 0.0
+    return {"bound": "hbm", "kernel": kernel, "algorithmic_bytes": algorithmic_bytes,
+            "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, **extra}
 
 
 def time_launches(fn, iters, warmup=2):
@@ -143,7 +193,7 @@ class Chain:
         self.buf.destroy()
 
 
-def measure_chain(ch, steps, warmup):
+def measure_chain(ch, steps, warmup, kernels=True):
     """W warm-up steps, then exactly K timed steps.  The K steps (plan, dispatch,
     combine on the rotating buffer sets) are recorded into one HIP graph, as the
     reference's harness does (benchmarks/bench_comm.py:118-156: events around one
@@ -190,6 +240,10 @@ def measure_chain(ch, steps, warmup):
     skip = min(2, steps - 1)
     in_chain = [sum(e[q].elapsed_time(e[q + 1]) for e in evs[skip:]) * 1e3 / (steps - skip) for q in range(3)]
     per = {}
+    per["single_replay_ms"] = single_ms
+    per["plan_us_in_chain"], per["dispatch_us_in_chain"], per["combine_us_in_chain"] = in_chain
+    if not kernels:      # the sweep only needs the chain and its kernels as they run in it
+        return wall_ms, ev_ms, per
     n = max(steps, 10)
     per["plan_us"] = time_launches(ch.plan_fn, n)
     k = [0]
@@ -319,7 +373,7 @@ def gpu_plan_all_ranks(S, K, E, R, tp, topk, tpe):
     return out
 
 
-def bench_weights(seed, steps):
+def bench_weights(seed, steps, cpu=True):
     """prefetch_weight (3 projections, one launch) and reduce_grad (one projection) at
     H=7168, H'=2048, epn=32, R=8 for two slot tables: the planner's own at maxvio~1
     (busiest owner) and a denser ring (every rank hosts 8 remote experts)."""
@@ -356,7 +410,8 @@ def bench_weights(seed, steps):
         by = 3 * (active + n_slots) * per * 2   # each owned expert read once, every slot written
         res[name] = {"rank": rank, "slots": n_slots, "active_experts": active,
                      "own_occupied_slots": own_slots, "prefetch_us_3proj": us,
-                     "prefetch_bytes": by, "prefetch_GBps": by / us / 1e3 if by else 0.0}
+                     "prefetch_bytes": by, "prefetch_GBps": by / us / 1e3 if by else 0.0,
+                     "prefetch_roofline": hbm_roofline("prefetch_kernel", by, us)}
     del local, pool
     torch.cuda.empty_cache()
     grad = torch.zeros(epn, H, Hp, dtype=torch.float32, device=dev)
@@ -365,9 +420,12 @@ def bench_weights(seed, steps):
         us = time_launches(lambda: launch_grad_reduce(grad, red, etc, rank=rank), steps)
         by = (n_slots + 2 * active + own_slots) * per * 4   # slots read, grads read+written, clears
         res[name].update({"grad_reduce_us": us, "grad_reduce_bytes": by,
-                          "grad_reduce_GBps": by / us / 1e3 if by else 0.0})
+                          "grad_reduce_GBps": by / us / 1e3 if by else 0.0,
+                          "grad_reduce_roofline": hbm_roofline("grad_reduce_kernel", by, us)})
     del grad, red
     torch.cuda.empty_cache()
+    if not cpu:
+        return res
     # host-core figures on a bounded sample of one projection: 16 slot copies
     # (index_copy_) and 8 slot sums (add_ then zero_), all torch threads; a 1 GiB
     # fill between warm-up and timing pushes the sample out of the host caches
@@ -438,8 +496,64 @@ def bench_ffn(seed, steps):
     }
 
 
+def write_traffic(fetch_csv, write_csv):
+    """profiles/traffic.json from the counter CSVs of two rocprofv3 --pmc runs of
+    `bench.py --profile-kernels` (one with FETCH_SIZE, one with WRITE_SIZE)."""
+    import csv
+
+    def per_kernel(path, counter):
+        acc = {}
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] != counter:
+                    continue
+                key = row["Kernel_Name"]
+                v = acc.setdefault(key, {"sum": 0.0, "n": 0, "grid": int(row["Grid_Size"]),
+                                         "wg": int(row["Workgroup_Size"])})
+                v["sum"] += float(row["Counter_Value"])
+                v["n"] += 1
+        return {k: (v["sum"] / v["n"], v["grid"] // v["wg"], v["n"]) for k, v in acc.items()}
+
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    copy = [k for k in fetch if "copyBuffer" in k]
+    assert copy, "the run must contain the 512 MiB copy the counters are scaled by"
+    known_kib = 512 * 1024
+    f_scale = known_kib / max(v[0] for k, v in fetch.items() if k in copy)
+    w_scale = known_kib / max(v[0] for k, v in write.items() if k in copy)
+    kernels = {}
+    for short in ("dispatch_kernel", "combine_kernel", "plan_kernel"):
+        names = [k for k in fetch if short in k]
+        if not names:
+            continue
+        k = names[0]
+        kernels[short] = {"name": k, "grid": fetch[k][1], "launches": fetch[k][2],
+                          "fetch_bytes": fetch[k][0] * 1024 * f_scale,
+                          "write_bytes": write[k][0] * 1024 * w_scale}
+    rec = {"source_digest": kernel_source_digest(),
+           "made_by": "python bench.py --write-traffic <fetch csv> <write csv> after two runs of "
+                      "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -- python3 bench.py --profile-kernels",
+           "scale": {"FETCH_SIZE": f_scale, "WRITE_SIZE": w_scale,
+                     "from": "a 512 MiB device-to-device copy in the same run"},
+           "workload": "config 1: S=4096 H=7168 K=8 E=256 R=8 token_padding=128 maxvio~1, rank 0",
+           "kernels": kernels}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    print(json.dumps(rec))
+
+
+def dispatch_grid(S, K, E, R, tp):
+    """Workgroups of one mep_dispatch launch (csrc/dispatch.hip: four (token, k) copies per
+    workgroup, then the zero-fill workgroups of 2*epn groups)."""
+    zpg = max(1, min(32, (tp - 1 + 3) // 4))
+    return (S * K + 3) // 4 + (2 * (E // R) * zpg if tp > 1 else 0)
+
+
 def main():
     args = parse()
+    if args.write_traffic:
+        write_traffic(*args.write_traffic)
+        return
     if args.gpus != 1:
         print("bench.py measures one rank's share on ONE GPU; --gpus > 1 is not part of this "
               "build (no collectives, no sharding).", file=sys.stderr)
@@ -462,9 +576,16 @@ def main():
     wall_ms, ev_ms, per = measure_chain(ch, args.steps, args.warmup)
     by = ch.bytes_one_way()
     value = 2 * by / (wall_ms * 1e-3) / 1e9
-    # roofline: the dominant kernel at its duration inside the timed steps
-    dom = "dispatch" if per["dispatch_us_in_chain"] >= per["combine_us_in_chain"] else "combine"
-    achieved = by / per[f"{dom}_us_in_chain"] / 1e3
+    # roofline: the dominant kernel, from its cold standalone duration (the duration inside
+    # the timed steps, with the tokens already pulled into cache by the planner launch, beside it)
+    dom = "dispatch" if per["dispatch_us"] >= per["combine_us"] else "combine"
+    grid = dispatch_grid(S, K, E, R, tp) if dom == "dispatch" else S * 7 // 4
+    traffic, traffic_note = measured_traffic(f"{dom}_kernel", grid)
+    roof = hbm_roofline(f"{dom}_kernel", by, per[f"{dom}_us"], traffic,
+                        duration_us=per[f"{dom}_us"], duration_us_in_timed_steps=per[f"{dom}_us_in_chain"],
+                        frac_in_timed_steps=by / per[f"{dom}_us_in_chain"] / 1e3 / HBM_PEAK_GBPS)
+    if traffic_note:
+        roof["traffic_note"] = traffic_note
     line = {
         "metric": "dispatch+combine GB/s of one rank's plan->dispatch->combine chain (plan us reported beside)",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -485,27 +606,36 @@ def main():
         "dispatch_us_warm_input": per["dispatch_us_warm_input"],
         "dispatch_pct_hbm_peak": 100.0 * per["dispatch_GBps"] / HBM_PEAK_GBPS,
         "combine_pct_hbm_peak": 100.0 * per["combine_GBps"] / HBM_PEAK_GBPS,
-        "roofline": {"bound": "hbm", "kernel": f"{dom}_kernel", "achieved": achieved,
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "algorithmic_bytes": by, "traffic": MEASURED_TRAFFIC_BYTES[dom]},
+        "roofline": roof,
+        "combine_roofline": hbm_roofline("combine_kernel", by, per["combine_us"],
+                                         measured_traffic("combine_kernel", S * 7 // 4)[0]),
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(ch)
     ch.destroy()
     torch.cuda.empty_cache()
-    if args.full:
+    if not args.chain_only:
         sweep = {}
+        sub_steps = max(5, args.steps // 2)
         for shape in ((4096, 7168, 256), (8192, 4096, 128)):
+            chain_us = []
             for mv in (0.0, 0.5, 1.0, 2.0, 4.0):
                 c2 = Chain(shape[0], shape[1], K, shape[2], R, tp, rank, mv, args.seed)
-                w2, e2, p2 = measure_chain(c2, args.steps, args.warmup)
+                w2, e2, p2 = measure_chain(c2, sub_steps, 2, kernels=False)
+                b2 = c2.bytes_one_way()
                 sweep[f"S{shape[0]}_H{shape[1]}_E{shape[2]}_maxvio{mv}"] = {
-                    "maxvio": round(c2.maxvio, 3), "chain_us": w2 * 1e3, "plan_us": p2["plan_us"],
-                    "dispatch_us": p2["dispatch_us"], "combine_us": p2["combine_us"]}
+                    "maxvio": round(c2.maxvio, 3), "chain_us": w2 * 1e3,
+                    "GBps": 2 * b2 / w2 / 1e6, "pct_hbm_peak": 2 * b2 / w2 / 1e6 / HBM_PEAK_GBPS * 100.0,
+                    "plan_us_in_chain": p2["plan_us_in_chain"],
+                    "dispatch_us_in_chain": p2["dispatch_us_in_chain"],
+                    "combine_us_in_chain": p2["combine_us_in_chain"]}
+                chain_us.append(w2 * 1e3)
                 c2.destroy()
                 torch.cuda.empty_cache()
+            sweep[f"S{shape[0]}_H{shape[1]}_E{shape[2]}_spread_pct"] = \
+                100.0 * (max(chain_us) - min(chain_us)) / min(chain_us)
         line["maxvio_sweep"] = sweep
-        line["weights"] = bench_weights(args.seed, max(5, args.steps // 2))
+        line["weights"] = bench_weights(args.seed, max(5, args.steps // 2), cpu=not args.no_cpu)
         torch.cuda.empty_cache()
         line["ffn"] = bench_ffn(args.seed, max(5, args.steps // 2))
     print(json.dumps(line))
