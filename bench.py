@@ -18,8 +18,9 @@ already pulled the tokens into the last-level cache, is reported beside it.
 The same line carries the other configurations: the chain at maxvio 0 .. 4 on
 both shapes (`maxvio_sweep`), prefetch_weight and reduce_grad at
 [32, 7168, 2048] per rank for the planner's own slot table and for a table with
-8 slots per rank (`weights`), and the expert-side grouped FFN (`ffn`), each
-with its own `roofline` record.  `--chain-only` skips them.
+8 slots per rank (`weights`), the expert-side grouped FFN (`ffn`), each with its
+own `roofline` record, and the chain bounded to 32 .. 256 compute units
+(`chain_on_limited_cus`).  `--chain-only` skips them.
 
 The CPU baseline is the scalar C restatement of the same chain
 (oracle/mep_oracle.c), timed on the host next to the GPU.
@@ -279,6 +280,40 @@ def measure_chain(ch, steps, warmup, kernels=True):
     per["single_replay_ms"] = single_ms
     per["plan_us_in_chain"], per["dispatch_us_in_chain"], per["combine_us_in_chain"] = in_chain
     return wall_ms, ev_ms, per
+
+
+def chain_on_limited_cus(ch, steps):
+    """What the chain costs when it may only use N compute units (a CU-masked stream, what
+    Buffer(num_sms=N) launches on): the figure a caller needs who runs the expert GEMMs beside
+    it on the other CUs.  Eager launches, HIP events on that stream (the GPU needs more time per
+    step than the host needs to issue one, so the queue never runs dry)."""
+    import torch
+
+    from moonep_amd.api import _limited_stream
+
+    out = {}
+    by = ch.bytes_one_way()
+    for n in (32, 64, 128, 256):
+        _, st = _limited_stream(0, n)
+        st.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(st):
+            for i in range(2):
+                ch.plan_fn(i); ch.dispatch_fn(i); ch.combine_fn(i)
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+            t = [0.0, 0.0, 0.0]
+            for i in range(steps):
+                j = i % len(ch.hidden)
+                evs[0].record(); ch.plan_fn(j)
+                evs[1].record(); ch.dispatch_fn(j)
+                evs[2].record(); ch.combine_fn(j)
+                evs[3].record()
+                evs[3].synchronize()
+                for q in range(3):
+                    t[q] += evs[q].elapsed_time(evs[q + 1]) * 1e3 / steps
+        torch.cuda.current_stream().wait_stream(st)
+        out[f"{n}_cus"] = {"plan_us": t[0], "dispatch_us": t[1], "combine_us": t[2],
+                           "chain_us": sum(t), "GBps": 2 * by / sum(t) / 1e3}
+    return out
 
 
 def cpu_baseline(ch, budget_s=10.0):
@@ -610,6 +645,8 @@ def main():
         "combine_roofline": hbm_roofline("combine_kernel", by, per["combine_us"],
                                          measured_traffic("combine_kernel", S * 7 // 4)[0]),
     }
+    if not args.chain_only:
+        line["chain_on_limited_cus"] = chain_on_limited_cus(ch, max(5, args.steps // 2))
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(ch)
     ch.destroy()

@@ -57,6 +57,20 @@ extern "C" {
 int mep_version(void);
 const char* mep_strerror(int code);
 
+/*
+ * A stream whose kernels run on at most `num_cus` compute units (a CU mask on
+ * the stream's hardware queue: the low num_cus bits, which the runtime spreads
+ * evenly over the XCDs).  This is what Buffer(num_sms=N) of the reference asks
+ * for (moonep/api.py:438-451, README.md:13: communication on 32 SMs beside the
+ * expert GEMMs): every mep_* call takes a stream, so launching the path on such
+ * a stream bounds all of its kernels at once, whatever their grids.  Default
+ * priority.  mep_stream_cu_census records, per workgroup of a small probe
+ * kernel, which CU it ran on (XCC id << 16 | HW_ID bits 8..15): for checking.
+ */
+int mep_stream_create_limited(int num_cus, void** stream_out);
+int mep_stream_destroy(void* stream);
+int mep_stream_cu_census(uint32_t* out, int nblocks, void* stream);
+
 /* Bytes of device scratch mep_plan / mep_plan_ranks need for `nranks` ranks
  * planned in one call (0 when the planner tables fit in LDS). */
 size_t mep_plan_scratch_bytes(int S, int K, int E, int R, int nranks);

@@ -34,6 +34,9 @@ _sz = C.c_size_t
 _SIGNATURES = {
     "mep_version": (_i, []),
     "mep_strerror": (C.c_char_p, [_i]),
+    "mep_stream_create_limited": (_i, [_i, C.POINTER(_p)]),
+    "mep_stream_destroy": (_i, [_p]),
+    "mep_stream_cu_census": (_i, [_p, _i, _p]),
     "mep_plan_scratch_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "mep_plan": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),
     "mep_plan_warm": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p, _sz, _p]),

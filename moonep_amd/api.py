@@ -41,11 +41,15 @@ One GPU stands in for the R expert-parallel ranks.  What that changes:
   prologue + combine pair does, so outputs are bit-identical; the standalone
   kernels stay available as ``launch_dispatch_epilogue`` /
   ``launch_combine_prologue``;
+* ``num_sms`` given explicitly bounds every kernel of this Buffer to that many
+  compute units: the comm stream is created with a CU mask and all operators
+  (synchronous ones too, the caller's stream then waits for them) launch on
+  it -- the reference's "communication on 32 SMs beside the expert GEMMs".
+  Left at ``None`` the kernels use the whole GPU on the caller's stream;
 * ``inter_rank_sync`` selects whether a threaded world's rendezvous are taken;
-  ``enable_pdl``, ``num_sms`` and ``comm_stream_priority`` are validated like the
-  reference and otherwise have no effect (HIP kernels on one stream run back to
-  back; the kernels size their own grids; all streams stay at the default
-  priority).
+  ``enable_pdl`` and ``comm_stream_priority`` are validated like the reference
+  and otherwise have no effect (HIP kernels on one stream run back to back; all
+  streams stay at the default priority).
 """
 
 from __future__ import annotations
@@ -311,6 +315,30 @@ def _create_context(S: int, H: int, K: int, E: int, num_ep_ranks: int, num_sms=N
     return ctx
 
 
+_LIMITED_STREAMS: dict = {}
+_LIMITED_LOCK = threading.Lock()
+
+
+def _limited_stream(device: int, num_cus: int):
+    """(raw handle, torch stream) of THE stream of ``device`` that is bound to
+    ``num_cus`` compute units.  One per (device, num_cus), shared by the Buffers
+    that ask for it and kept until the process ends: torch's allocator remembers
+    every stream a tensor was recorded on (``record_stream``) and touches it again
+    when the tensor is freed, so such a stream must never be destroyed."""
+    import ctypes
+
+    from . import _lib
+    key = (int(device), int(num_cus))
+    with _LIMITED_LOCK:
+        if key not in _LIMITED_STREAMS:
+            handle = ctypes.c_void_p()
+            with torch.cuda.device(device):
+                _lib.check(_lib.lib().mep_stream_create_limited(num_cus, ctypes.byref(handle)),
+                           "mep_stream_create_limited")
+            _LIMITED_STREAMS[key] = (handle.value, torch.cuda.ExternalStream(handle.value, device=device))
+        return _LIMITED_STREAMS[key]
+
+
 class Buffer:
     """Owner of the communication buffers and the comm stream; see the module
     docstring for the differences to the reference."""
@@ -329,12 +357,18 @@ class Buffer:
         self.comm_stream_priority = comm_stream_priority
         self.enable_pdl = enable_pdl
         self._comm_stream = None
+        self._limited_stream = None      # raw handle of a CU-masked comm stream, if any
         self._destroyed = False
         self._ctx = _create_context(S, H, K, E, num_ep_ranks, num_sms=num_sms,
                                     token_padding=token_padding, group=group, rank=rank,
                                     world=world)
         # default priority on purpose: mixed stream priorities are not used on this hardware
-        self._comm_stream = torch.cuda.Stream(device=int(self._ctx["device"]))
+        if num_sms is None:
+            self._comm_stream = torch.cuda.Stream(device=int(self._ctx["device"]))
+        else:
+            # an explicit num_sms: every kernel of this Buffer runs on that many CUs
+            self._limited_stream, self._comm_stream = _limited_stream(
+                int(self._ctx["device"]), int(self._ctx["num_sms"]))
 
     # -- lifecycle -----------------------------------------------------------
     @property
@@ -369,6 +403,7 @@ class Buffer:
             self._ctx.clear()
         self._ctx = None
         self._comm_stream = None
+        self._limited_stream = None      # the stream itself stays (see _limited_stream)
         self._destroyed = True
 
     def __del__(self):
@@ -396,6 +431,20 @@ class Buffer:
     def _plan_runtime_tensors(plan: MoonEPCommPlan):
         return (plan.dst, plan.experts_to_copy, plan.zero_fill_ranges, plan.remote_stats,
                 plan.dup_groups, plan.dup_loffs, plan.dup_counts)
+
+    def _finish(self, tensors, fn, async_finish: bool):
+        """Run an operator body: directly on the caller's stream, or -- when the
+        result is wanted asynchronously or the Buffer is bound to ``num_sms`` CUs --
+        on the comm stream.  Returns the completion event for ``async_finish``,
+        else None (the caller's stream then already waits for the work)."""
+        if not async_finish and self._limited_stream is None:
+            fn()
+            return None
+        done = self._on_comm_stream(tensors, fn)
+        if async_finish:
+            return done
+        torch.cuda.current_stream().wait_event(done)
+        return None
 
     def _on_comm_stream(self, tensors, fn):
         """Run ``fn`` on the comm stream after the current stream's work and
@@ -533,14 +582,13 @@ class Buffer:
                                route_weights_nvs, zero_copy, router_weights_zero_copy,
                                bool(inter_rank_sync))
 
-        if not async_finish:
-            run()
-            return hidden_nvsh, route_weights_nvs, cu_seqlens, plan
         tensors = [hidden_sh, route_weights_sk, hidden_nvsh, route_weights_nvs,
                    *self._plan_runtime_tensors(plan)]
         if planning_args is not None:
             tensors.extend(planning_args)
-        done = self._on_comm_stream(tensors, run)
+        done = self._finish(tensors, run, async_finish)
+        if not async_finish:
+            return hidden_nvsh, route_weights_nvs, cu_seqlens, plan
         return hidden_nvsh, route_weights_nvs, cu_seqlens, plan, done
 
     def prefetch_weight(self, plan: MoonEPCommPlan | None = None, async_finish: bool = False, *,
@@ -590,11 +638,8 @@ class Buffer:
                             rank=int(ctx["rank"]), num_sms=int(ctx["num_sms"]))
             ctx["world"].rendezvous(int(ctx["rank"]))   # every owner has pushed into every pool
 
-        if not async_finish:
-            run()
-            return None
         extra = (*local_scales, *scale_pools) if scales else ()
-        return self._on_comm_stream((plan.experts_to_copy, *local_weights, *pools, *extra), run)
+        return self._finish((plan.experts_to_copy, *local_weights, *pools, *extra), run, async_finish)
 
     def combine(self, plan: MoonEPCommPlan | None = None, hidden_nvsh=None, route_weights_nvs=None,
                 async_finish: bool = False, inter_rank_sync: bool = True, *,
@@ -637,12 +682,9 @@ class Buffer:
                               route_weights_sk, zero_copy, router_weights_zero_copy,
                               bool(inter_rank_sync))
 
-        if not async_finish:
-            run()
-            return hidden_sh, route_weights_sk, None
-        done = self._on_comm_stream(
+        done = self._finish(
             (hidden_sh, *self._plan_runtime_tensors(plan), hidden_nvsh, route_weights_nvs,
-             route_weights_sk), run)
+             route_weights_sk), run, async_finish)
         return hidden_sh, route_weights_sk, done
 
     def reduce_grad(self, plan: MoonEPCommPlan | None = None, async_finish: bool = False, *,
@@ -685,7 +727,4 @@ class Buffer:
                 launch_grad_reduce(local, pool, plan.experts_to_copy, rank=rank,
                                    num_sms=int(ctx["num_sms"]), phase="clear")
 
-        if not async_finish:
-            run()
-            return None
-        return self._on_comm_stream((plan.experts_to_copy, *local_grads, *pools), run)
+        return self._finish((plan.experts_to_copy, *local_grads, *pools), run, async_finish)

@@ -1,5 +1,8 @@
-// Version and error strings of the C ABI.
+// Version and error strings of the C ABI, and the CU-limited stream behind
+// Buffer(num_sms=...).
 #include "mep_common.h"
+
+#include <vector>
 
 extern "C" int mep_version(void) { return 100; }  // major*10000 + minor*100 + patch
 
@@ -17,4 +20,46 @@ extern "C" const char* mep_strerror(int code) {
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "unknown error";
+}
+
+namespace {
+
+// one record per workgroup: XCC id in bits 16..19, the SE / SH / CU fields of HW_ID in bits 8..15
+__global__ void cu_census_kernel(uint32_t* out) {
+  if (threadIdx.x == 0) {
+    uint32_t hw, xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    out[blockIdx.x] = ((xcc & 0xfu) << 16) | (hw & 0xff00u);
+  }
+}
+
+}  // namespace
+
+extern "C" int mep_stream_create_limited(int num_cus, void** stream_out) {
+  MEP_REQUIRE(stream_out, MEP_ERR_INVALID_ARG);
+  int dev = 0, cus = 0;
+  MEP_RETURN_IF_HIP(hipGetDevice(&dev));
+  MEP_RETURN_IF_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  MEP_REQUIRE(num_cus >= 1 && num_cus <= cus, MEP_ERR_INVALID_ARG);
+  // The low num_cus bits: the runtime spreads consecutive bits over the XCDs (32 bits = 4 CUs on
+  // each of 8 XCDs).  Only such contiguous masks are used: they were run from 16 to 256 CUs.
+  std::vector<uint32_t> mask((size_t)(cus + 31) / 32, 0u);
+  for (int i = 0; i < num_cus; ++i) mask[i / 32] |= 1u << (i % 32);
+  hipStream_t st = nullptr;
+  MEP_RETURN_IF_HIP(hipExtStreamCreateWithCUMask(&st, (uint32_t)mask.size(), mask.data()));
+  *stream_out = (void*)st;
+  return MEP_OK;
+}
+
+extern "C" int mep_stream_destroy(void* stream) {
+  MEP_REQUIRE(stream, MEP_ERR_INVALID_ARG);
+  MEP_RETURN_IF_HIP(hipStreamDestroy((hipStream_t)stream));
+  return MEP_OK;
+}
+
+extern "C" int mep_stream_cu_census(uint32_t* out, int nblocks, void* stream) {
+  MEP_REQUIRE(out && nblocks > 0, MEP_ERR_INVALID_ARG);
+  hipLaunchKernelGGL(cu_census_kernel, dim3(nblocks), dim3(64), 0, (hipStream_t)stream, out);
+  return mep_launch_status();
 }
