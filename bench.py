@@ -82,6 +82,9 @@ def parse():
                     help="no GPU work: turn the counter_collection.csv files of two rocprofv3 --pmc runs of "
                          "`bench.py --profile-kernels` (FETCH_SIZE, WRITE_SIZE) into profiles/traffic.json")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-limited-cus", action="store_true",
+                    help="skip the leg that times the chain on CU-masked streams (under rocprofv3 a process "
+                         "that still holds such a stream has crashed in the profiler's exit handlers)")
     ap.add_argument("--profile-kernels", action="store_true",
                     help="for rocprofv3: a few plain launches of each kernel and of a 512 MiB "
                          "torch copy (the known-size kernel counters are scaled by); no JSON")
@@ -542,7 +545,9 @@ def write_traffic(fetch_csv, write_csv):
             for row in csv.DictReader(f):
                 if row["Counter_Name"] != counter:
                     continue
-                key = row["Kernel_Name"]
+                # launches of one kernel with another grid (the runtime's small staging copies
+                # share the name of the 512 MiB copy) are records of their own
+                key = (row["Kernel_Name"], int(row["Grid_Size"]))
                 v = acc.setdefault(key, {"sum": 0.0, "n": 0, "grid": int(row["Grid_Size"]),
                                          "wg": int(row["Workgroup_Size"])})
                 v["sum"] += float(row["Counter_Value"])
@@ -550,18 +555,18 @@ def write_traffic(fetch_csv, write_csv):
         return {k: (v["sum"] / v["n"], v["grid"] // v["wg"], v["n"]) for k, v in acc.items()}
 
     fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
-    copy = [k for k in fetch if "copyBuffer" in k]
+    copy = [k for k in fetch if "copyBuffer" in k[0]]
     assert copy, "the run must contain the 512 MiB copy the counters are scaled by"
     known_kib = 512 * 1024
     f_scale = known_kib / max(v[0] for k, v in fetch.items() if k in copy)
     w_scale = known_kib / max(v[0] for k, v in write.items() if k in copy)
     kernels = {}
     for short in ("dispatch_kernel", "combine_kernel", "plan_kernel"):
-        names = [k for k in fetch if short in k]
+        names = [k for k in fetch if short in k[0]]
         if not names:
             continue
         k = names[0]
-        kernels[short] = {"name": k, "grid": fetch[k][1], "launches": fetch[k][2],
+        kernels[short] = {"name": k[0], "grid": fetch[k][1], "launches": fetch[k][2],
                           "fetch_bytes": fetch[k][0] * 1024 * f_scale,
                           "write_bytes": write[k][0] * 1024 * w_scale}
     rec = {"source_digest": kernel_source_digest(),
@@ -645,7 +650,7 @@ def main():
         "combine_roofline": hbm_roofline("combine_kernel", by, per["combine_us"],
                                          measured_traffic("combine_kernel", S * 7 // 4)[0]),
     }
-    if not args.chain_only:
+    if not (args.chain_only or args.no_limited_cus):
         line["chain_on_limited_cus"] = chain_on_limited_cus(ch, max(5, args.steps // 2))
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(ch)
