@@ -500,6 +500,7 @@ def bench_ffn(seed, steps):
     import torch
 
     from moonep_amd import routing
+    from moonep_amd import ffn
     from moonep_amd.ffn import launch_grouped_gemm_nt
 
     S, K, E, R, H, Hp = 4096, 8, 256, 8, 7168, 2048
@@ -524,8 +525,37 @@ def bench_ffn(seed, steps):
     c = torch.empty(used, Hp, dtype=torch.bfloat16, device=dev)
     t3 = time_launches(lambda: torch.matmul(rows[:used], gate[0].t(), out=c), steps)
     peak = 2500.0
+    # backward of the same FFN: every GEMM on the grouped kernel; the transposes that give the
+    # operands their other orientation are timed with it
+    del c
+    dy = torch.randn(NvS, H, device=dev, generator=g).to(torch.bfloat16)
+    _, saved = ffn.grouped_ffn_hip_forward(rows, slots, cu, gate, up, down)
+    bw = {}
+    down_t = ffn.transpose_bf16(down)
+    bw["transpose_weights_us"] = 3 * time_launches(lambda: ffn.transpose_bf16(down, down_t), max(2, steps // 2))
+    dh = launch_grouped_gemm_nt(dy, down_t, cu)
+    bw["dh_gemm_us"] = time_launches(lambda: launch_grouped_gemm_nt(dy, down_t, cu, dh), steps)
+    del down_t
+    sb = ffn.launch_swiglu_bwd(dh, saved[0], saved[1], slots, cu)
+    dg, du = sb[0], sb[1]
+    bw["swiglu_bwd_us"] = time_launches(lambda: ffn.launch_swiglu_bwd(dh, saved[0], saved[1], slots, cu, sb), steps)
+    gate_n, up_n = ffn.transpose_bf16(gate), ffn.transpose_bf16(up)
+    drows = ffn.launch_grouped_gemm_dual_nt(dg, gate_n, du, up_n, cu)
+    bw["dual_dgrad_gemm_us"] = time_launches(
+        lambda: ffn.launch_grouped_gemm_dual_nt(dg, gate_n, du, up_n, cu, drows), steps)
+    del gate_n, up_n, drows
+    rows_t, dg_t = ffn.transpose_bf16(rows), ffn.transpose_bf16(dg)
+    bw["transpose_activations_us"] = (2 * time_launches(lambda: ffn.transpose_bf16(rows, rows_t), steps)
+                                      + 3 * time_launches(lambda: ffn.transpose_bf16(dg, dg_t), steps))
+    dwg = ffn.launch_grouped_gemm_wgrad(dg_t, rows_t, cu)
+    bw["wgrad_gemm_us_each"] = time_launches(lambda: ffn.launch_grouped_gemm_wgrad(dg_t, rows_t, cu, dwg), steps)
+    del rows_t, dg_t, dg, du, sb, dh, dwg
+    gemm_us = bw["dh_gemm_us"] + bw["dual_dgrad_gemm_us"] + 3 * bw["wgrad_gemm_us_each"]
+    bw["gemm_TFLOPs"] = 12.0 * used * H * Hp / gemm_us / 1e6
+    bw["total_us"] = gemm_us + bw["swiglu_bwd_us"] + bw["transpose_weights_us"] + bw["transpose_activations_us"]
+    bw["TFLOPs_with_transposes"] = 12.0 * used * H * Hp / bw["total_us"] / 1e6
     return {
-        "rows_in_groups": used, "NvS": NvS, "groups": G, "maxvio": mv,
+        "rows_in_groups": used, "NvS": NvS, "groups": G, "maxvio": mv, "backward": bw,
         "swiglu_gate_up_us": t1, "swiglu_gate_up_TFLOPs": f1 / t1 / 1e6,
         "down_us": t2, "down_TFLOPs": f2 / t2 / 1e6,
         "roofline": {"bound": "mfma", "kernel": "grouped_gemm_nt_kernel", "achieved": (f1 + f2) / (t1 + t2) / 1e6,

@@ -237,6 +237,58 @@ int mep_grouped_gemm_nt(const void* A, const void* B, const void* B_up, const in
                         int G, void* C, const float* row_scale, int M, int N, int K, int swiglu,
                         void* stream);
 
+/*
+ * The same fused gate/up GEMM, storing the two pre-activations beside the
+ * activation for a backward pass: C_act = bf16(silu(g) * u), C_gate = bf16(g),
+ * C_up = bf16(u), g = A*B_gate[g]^T, u = A*B_up[g]^T.  C_gate / C_up may be
+ * NULL.  No counterpart in the reference (the expert FFN is the caller's).
+ */
+int mep_grouped_swiglu_nt(const void* A, const void* B_gate, const void* B_up,
+                          const int32_t* cu_seqlens, int G, void* C_act, void* C_gate, void* C_up,
+                          int M, int N, int K, void* stream);
+
+/*
+ * C = bf16(A1 * B1[g]^T + A2 * B2[g]^T), one K loop over both pairs: the input
+ * gradient of the gate/up pair (A1 = d gate, B1 = gate weights [G,N,K] with K
+ * the hidden width of the experts, likewise the up pair).  Shapes as
+ * mep_grouped_gemm_nt without swiglu.  No counterpart in the reference.
+ */
+int mep_grouped_gemm_dual_nt(const void* A1, const void* B1, const void* A2, const void* B2,
+                             const int32_t* cu_seqlens, int G, void* C, int M, int N, int K,
+                             void* stream);
+
+/*
+ * Weight gradients of the grouped GEMMs from TRANSPOSED activations:
+ * C[g] [Ma,Nb] fp32 = At[:, rows of g] * Bt[:, rows of g]^T, At [Ma,ld] and
+ * Bt [Nb,ld] bf16 with the rank's rows along the contiguous dimension; the rows
+ * of group g are [cu_seqlens[g-1], cu_seqlens[g]).  A group without rows gets
+ * zeros.  Ma % 128 == 0, Nb % 256 == 0, ld % 128 == 0, ld >= cu_seqlens[G-1].
+ * The fp32 [G,Ma,Nb] result has the layout mep_grad_reduce sums (local experts
+ * first, then the slots).  No counterpart in the reference.
+ */
+int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int32_t* cu_seqlens, int G,
+                           float* C, int Ma, int Nb, int64_t ld, void* stream);
+
+/*
+ * [batch, rows, cols] -> [batch, cols, rows] of bf16 (any 2-byte element);
+ * rows % 64 == 0, cols % 64 == 0, src != dst.  Feeds mep_grouped_gemm_wgrad
+ * and the backward GEMMs, which want the other operand orientation.
+ */
+int mep_transpose_bf16(const void* src, void* dst, int batch, int rows, int cols, void* stream);
+
+/*
+ * Backward of the SwiGLU activation with the route weight applied,
+ * h = s * silu(g) * u, from dh' = dy * W_down (gradient of the unscaled
+ * activation), all [M,N] bf16, row_scale s [M] fp32 or NULL:
+ *   dgate = s*dh' * u * silu'(g), dup = s*dh' * silu(g), hs = s * silu(g) * u
+ *   (the operand of the down projection's weight gradient),
+ *   dscale[m] = sum_n dh'[m,n] * silu(g)*u  (fp32, may be NULL).
+ * Rows at or beyond cu_seqlens[G-1] come out as zeros.  N % 8 == 0.
+ */
+int mep_swiglu_bwd(const void* dh, const void* gate_pre, const void* up_pre, const float* row_scale,
+                   const int32_t* cu_seqlens, int G, void* dgate, void* dup, void* hs, float* dscale,
+                   int M, int N, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

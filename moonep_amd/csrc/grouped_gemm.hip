@@ -11,10 +11,16 @@
 // multiple of 128 a row tile never straddles two groups.  The kernel is bound
 // by the L2 (its channels are ~75 % busy at 0.8 PFLOP/s), i.e. by tile bytes
 // per flop.
-// Two epilogues:
+// Four kinds of launch share the main loop:
 //   scale  : C[m,n] = bf16(row_scale[m] * acc)               (down projection)
 //   swiglu : C[m,n] = bf16(silu(A*Bg^T) * (A*Bu^T))           (gate/up fused;
-//            the tile holds 128 gate rows and the same 128 up rows)
+//            the tile holds 128 gate rows and the same 128 up rows; the two
+//            pre-activations can be stored beside it for the backward pass)
+//   dual   : C = bf16(A*B[g]^T + A2*B2[g]^T): the K loop runs over both pairs
+//            (input gradient of the gate/up pair)
+//   wgrad  : C[g] = At[:, rows of g] * Bt[:, rows of g]^T in fp32: the K range
+//            of a tile is the row range of its group (weight gradients from
+//            transposed activations)
 // Tiles are handed out so that the workgroups running at one time on an XCD
 // (one L2) work on the same 8 row tiles and neighbouring weight tiles.
 #include "mep_common.h"
@@ -46,7 +52,14 @@ struct GemmArgs {
   uint16_t* C;         // [M,N]
   const float* scale;  // [M] or null
   int M, N, K, G, mtiles, ntiles;
+  const uint16_t* A2;  // dual: rows of the second K segment [M,K]
+  uint16_t* Cg;        // swiglu: gate pre-activation [M,N] or null
+  uint16_t* Cu;        // swiglu: up pre-activation [M,N] or null
+  float* Cf;           // wgrad: [G,M,N] fp32
+  int64_t ld;          // row stride of A and B in elements (K, or the row count for wgrad)
 };
+
+enum { kModeScale = 0, kModeSwiglu = 1, kModeDual = 2, kModeWgrad = 3 };
 
 __device__ __forceinline__ float mep_silu(float x) { return x / (1.0f + __expf(-x)); }
 
@@ -64,18 +77,22 @@ __device__ __forceinline__ void mep_wait_vmcnt() {
 // back to the producers.  A stage row is the bare 128-byte slice; the 16-byte
 // vector q of row r sits at position q ^ (r & 7), so the eight rows a group of
 // eight lanes reads fall into distinct banks.
-template <bool SWIGLU>
+template <int MODE>
 __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmArgs a) {
+  constexpr bool SWIGLU = MODE == kModeSwiglu;
   extern __shared__ __attribute__((aligned(1024))) char gsm[];
   __shared__ int s_group;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   // ---- which tile: XCD x (workgroups x, x+8, ...) walks a contiguous range of
   // tiles; inside a panel of kPanel row tiles the row tile index runs fastest
-  const int total = a.mtiles * a.ntiles;
+  const int per_group = a.mtiles * a.ntiles;
+  const int total = MODE == kModeWgrad ? per_group * a.G : per_group;
   const int per_xcd = (total + 7) >> 3;
-  const int L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (L >= total) return;
+  const int L0 = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (L0 >= total) return;
+  const int tg = MODE == kModeWgrad ? L0 / per_group : 0;  // wgrad: the group is part of the tile index
+  const int L = L0 - tg * per_group;
   const int panel = L / (kPanel * a.ntiles);
   const int within = L - panel * (kPanel * a.ntiles);
   const int ph = min(kPanel, a.mtiles - panel * kPanel);
@@ -86,7 +103,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   const int n0 = nt * kCols;
 
   // ---- group of this row tile: the first whose padded end lies beyond m0
-  if (wave == 0) {
+  if (MODE == kModeWgrad) {
+    if (tid == 0) s_group = tg;
+  } else if (wave == 0) {
     int g = -1;
     for (int c = 0; c < a.G && g < 0; c += 64) {
       const int end = c + lane < a.G ? a.cu[c + lane] : 0;
@@ -99,8 +118,15 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   const int g = s_group;
   if (g < 0) return;  // rows past the last group: nothing to compute
 
-  const int KT = a.K / kBK;
-  const size_t K = (size_t)a.K;
+  // K steps of this tile and where its K range starts in a row
+  int kbeg = 0, KT = a.K / kBK;
+  if (MODE == kModeDual) KT *= 2;
+  if (MODE == kModeWgrad) {
+    kbeg = g > 0 ? a.cu[g - 1] : 0;
+    KT = (a.cu[g] - kbeg) / kBK;
+  }
+  const size_t K = (size_t)a.ld;
+  const bool any = KT > 0;  // a group without rows: its weight gradient is zero
 
   if (wave >= kConsumers) {
     // =============================== producer ===============================
@@ -109,19 +135,30 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
     // piece j of a stage: rows 8j .. 8j+7 of the row tile (j < 16), then of the
     // weight tile; this wave moves the pieces j = p, p + kProducers, ...
     // lane (r, kv) fetches vector kv ^ r of its row into slot (r, kv)
-    const uint16_t* Ap = a.A + (size_t)(m0 + r) * K + ((kv ^ r) * 8);
-    const uint16_t* Bp0 = a.B + (size_t)g * a.N * K + (size_t)(n0 + r) * K + ((kv ^ r) * 8);
-    const uint16_t* Bp1 = SWIGLU ? a.B2 + (size_t)g * a.N * K + (size_t)(n0 + r) * K + ((kv ^ r) * 8)
-                                 : Bp0 + (size_t)(kBN / 2) * K;
+    if (!any) return;
+    const size_t goff = MODE == kModeWgrad ? (size_t)kbeg : (size_t)g * a.N * K;
+    const size_t lane_off = (size_t)r * K + ((kv ^ r) * 8);
+    const uint16_t* Ap = a.A + (size_t)m0 * K + lane_off + (MODE == kModeWgrad ? (size_t)kbeg : 0);
+    const uint16_t* Bp0 = a.B + goff + (size_t)n0 * K + lane_off;
+    const uint16_t* Bp1 = SWIGLU ? a.B2 + goff + (size_t)n0 * K + lane_off : Bp0 + (size_t)(kBN / 2) * K;
+    // dual: the second half of the K loop reads the second pair
+    const uint16_t* Aq = MODE == kModeDual ? a.A2 + (size_t)m0 * K + lane_off : Ap;
+    const uint16_t* Bq0 = MODE == kModeDual ? a.B2 + goff + (size_t)n0 * K + lane_off : Bp0;
+    const uint16_t* Bq1 = Bq0 + (size_t)(kBN / 2) * K;
     auto issue = [&](int k0, int stage) {
       char* base = gsm + stage * kStage;
+      const bool second = MODE == kModeDual && k0 >= a.K;
+      if (second) k0 -= a.K;
+      const uint16_t* pa = second ? Aq : Ap;
+      const uint16_t* pb0 = second ? Bq0 : Bp0;
+      const uint16_t* pb1 = second ? Bq1 : Bp1;
 #pragma unroll
       for (int q = 0; q < kPiecesPerProducer; ++q) {
         const int j = p + q * kProducers;  // 0 .. 47
         const uint16_t* src;
-        if (j < kBM / 8) src = Ap + (size_t)(8 * j) * K + k0;
-        else if (j < kBM / 8 + kBN / 16) src = Bp0 + (size_t)(8 * (j - kBM / 8)) * K + k0;
-        else src = Bp1 + (size_t)(8 * (j - kBM / 8 - kBN / 16)) * K + k0;
+        if (j < kBM / 8) src = pa + (size_t)(8 * j) * K + k0;
+        else if (j < kBM / 8 + kBN / 16) src = pb0 + (size_t)(8 * (j - kBM / 8)) * K + k0;
+        else src = pb1 + (size_t)(8 * (j - kBM / 8 - kBN / 16)) * K + k0;
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                          (__attribute__((address_space(3))) void*)(base + j * 1024),
                                          16, 0, 0);
@@ -162,8 +199,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   const int oa0 = arow * kRowBytes, oa1 = (arow + 32) * kRowBytes;
   const int ob0 = brow0 * kRowBytes, ob1 = brow1 * kRowBytes;
 
-  __builtin_amdgcn_s_barrier();  // stage 0 is filled
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  if (any) {
+    __builtin_amdgcn_s_barrier();  // stage 0 is filled
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  }
   int st = 0;
   for (int kt = 0; kt < KT; ++kt) {
     const char* sb = gsm + st * kStage;
@@ -188,6 +227,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   // ---- epilogue.  acc[i][j][v]: row 64*wm + 32*i + 8*(v/4) + 4*(lane/32) + v%4,
   // column (lane % 32) of the j-th 32-wide block
   const int ldc = a.N;
+  float* cf = MODE == kModeWgrad ? a.Cf + (size_t)g * a.M * a.N : nullptr;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -197,6 +237,12 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
         const int n = n0 + 32 * wn + (lane & 31);
         const float res = mep_silu(acc[i][0][v]) * acc[i][1][v];
         a.C[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(res);
+        if (a.Cg) a.Cg[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(acc[i][0][v]);
+        if (a.Cu) a.Cu[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(acc[i][1][v]);
+      } else if (MODE == kModeWgrad) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          cf[(size_t)m * ldc + n0 + 64 * wn + 32 * j + (lane & 31)] = acc[i][j][v];
       } else {
         const float sc = a.scale ? a.scale[m] : 1.0f;
 #pragma unroll
@@ -208,49 +254,230 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
     }
 }
 
+// ---------------------------------------------------------------------------
+// [batch, rows, cols] -> [batch, cols, rows] of 2-byte elements through a
+// 64 x 64 LDS tile (rows and cols multiples of 64): 128-byte reads and writes.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* __restrict__ src,
+                                                          uint16_t* __restrict__ dst, int rows, int cols) {
+  __shared__ uint16_t tile[64][66];
+  const size_t plane = (size_t)rows * cols;
+  const uint16_t* s = src + (size_t)blockIdx.z * plane;
+  uint16_t* d = dst + (size_t)blockIdx.z * plane;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8 threads, two columns each
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = ty + 8 * i;
+    const uint32_t v = *(const uint32_t*)(s + (size_t)(r0 + r) * cols + c0 + 2 * tx);
+    tile[r][2 * tx] = (uint16_t)v;
+    tile[r][2 * tx + 1] = (uint16_t)(v >> 16);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = ty + 8 * i;  // column of the source = row of the destination
+    const uint32_t v = (uint32_t)tile[2 * tx][c] | ((uint32_t)tile[2 * tx + 1][c] << 16);
+    *(uint32_t*)(d + (size_t)(c0 + c) * rows + r0 + 2 * tx) = v;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward of h = s * silu(g) * u per element, from the gradient dh' of the
+// unscaled activation (dh' = dy * Wdown):
+//   dgate = s*dh' * u * silu'(g),  dup = s*dh' * silu(g),  hs = s * silu(g) * u,
+//   dscale[m] = sum_n dh'[m,n] * silu(g)*u
+// One wave per row; rows at or beyond cu_seqlens[G-1] come out as zeros.
+// ---------------------------------------------------------------------------
+struct SwigluBwdArgs {
+  const uint16_t* dh; const uint16_t* gate; const uint16_t* up; const float* scale; const int* cu;
+  uint16_t* dgate; uint16_t* dup; uint16_t* hs; float* dscale;
+  int M, N, G;
+};
+
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(SwigluBwdArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int m = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (m >= a.M) return;
+  const bool live = m < a.cu[a.G - 1];
+  const float s = a.scale ? a.scale[m] : 1.0f;
+  const size_t row = (size_t)m * a.N;
+  float dot = 0.0f;
+  for (int n = lane * 8; n < a.N; n += 512) {
+    uint4 od = make_uint4(0, 0, 0, 0), og = od, oh = od;
+    if (live) {
+      const uint4 vd = *(const uint4*)(a.dh + row + n);
+      const uint4 vg = *(const uint4*)(a.gate + row + n);
+      const uint4 vu = *(const uint4*)(a.up + row + n);
+      const uint32_t wd[4] = {vd.x, vd.y, vd.z, vd.w}, wg[4] = {vg.x, vg.y, vg.z, vg.w},
+                     wu[4] = {vu.x, vu.y, vu.z, vu.w};
+      uint32_t rg[4], ru[4], rh[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float fg[2], fu[2], fh[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const float d = e ? mep_bf16_hi(wd[q]) : mep_bf16_lo(wd[q]);
+          const float g = e ? mep_bf16_hi(wg[q]) : mep_bf16_lo(wg[q]);
+          const float u = e ? mep_bf16_hi(wu[q]) : mep_bf16_lo(wu[q]);
+          const float sig = 1.0f / (1.0f + __expf(-g));
+          const float act = g * sig;               // silu(g)
+          dot += d * act * u;
+          const float dhs = s * d;                 // gradient of the scaled activation
+          fg[e] = dhs * u * (sig + act * (1.0f - sig));
+          fu[e] = dhs * act;
+          fh[e] = s * act * u;
+        }
+        rg[q] = mep_pack_bf16(fg[0], fg[1]);
+        ru[q] = mep_pack_bf16(fu[0], fu[1]);
+        rh[q] = mep_pack_bf16(fh[0], fh[1]);
+      }
+      od = make_uint4(rg[0], rg[1], rg[2], rg[3]);
+      og = make_uint4(ru[0], ru[1], ru[2], ru[3]);
+      oh = make_uint4(rh[0], rh[1], rh[2], rh[3]);
+    }
+    *(uint4*)(a.dgate + row + n) = od;
+    *(uint4*)(a.dup + row + n) = og;
+    *(uint4*)(a.hs + row + n) = oh;
+  }
+  if (a.dscale) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) dot += __shfl_xor(dot, d);
+    if (lane == 0) a.dscale[m] = dot;
+  }
+}
+
+// 144 KB of dynamic LDS needs the opt-in, once per device and kernel
+template <int MODE>
+int gemm_launch(const GemmArgs& a, int64_t total, hipStream_t st) {
+  MEP_REQUIRE(total > 0 && total < (1 << 30), MEP_ERR_UNSUPPORTED);
+  const int per_xcd = (int)((total + 7) / 8);
+  const size_t lds = (size_t)kStages * kStage;
+  static std::atomic<uint64_t> opted{0};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (!(opted.load(std::memory_order_acquire) & bit)) {
+    e = hipFuncSetAttribute((const void*)grouped_gemm_nt_kernel<MODE>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    opted.fetch_or(bit, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(grouped_gemm_nt_kernel<MODE>, dim3(per_xcd * 8), dim3(kGemmThreads), lds, st, a);
+  return mep_launch_status();
+}
+
+int check_nt_shapes(const void* A, const void* B, const int32_t* cu, const void* C, int M, int N, int K,
+                    int G, int cols_per_tile) {
+  MEP_REQUIRE(A && B && cu && C, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(M > 0 && N > 0 && K > 0 && G > 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(M % kBM == 0 && K % kBK == 0 && N % cols_per_tile == 0, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((int64_t)M * (N > K ? N : K) < ((int64_t)1 << 40), MEP_ERR_UNSUPPORTED);
+  return MEP_OK;
+}
+
+GemmArgs nt_args(const void* A, const void* B, const void* B2, const int32_t* cu, void* C, const float* scale,
+                 int M, int N, int K, int G, int cols_per_tile) {
+  GemmArgs a{};
+  a.A = (const uint16_t*)A; a.B = (const uint16_t*)B; a.B2 = (const uint16_t*)B2;
+  a.cu = cu; a.C = (uint16_t*)C; a.scale = scale;
+  a.M = M; a.N = N; a.K = K; a.G = G;
+  a.mtiles = M / kBM;
+  a.ntiles = N / cols_per_tile;
+  a.ld = K;
+  return a;
+}
+
+int gemm_nt_forward(const void* A, const void* B, const void* B_up, const int32_t* cu, int G, void* C,
+                    void* C_gate, void* C_up, const float* row_scale, int M, int N, int K, int swiglu,
+                    void* stream) {
+  const int cols = swiglu ? kBN / 2 : kBN;
+  const int rc = check_nt_shapes(A, B, cu, C, M, N, K, G, cols);
+  if (rc != MEP_OK) return rc;
+  MEP_REQUIRE(!swiglu || (B_up && !row_scale), MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(swiglu || (!C_gate && !C_up), MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)B_up % 16 == 0) &&
+                  ((uintptr_t)C % 2 == 0) && ((uintptr_t)C_gate % 2 == 0) && ((uintptr_t)C_up % 2 == 0),
+              MEP_ERR_ALIGNMENT);
+  GemmArgs a = nt_args(A, B, B_up, cu, C, row_scale, M, N, K, G, cols);
+  a.Cg = (uint16_t*)C_gate;
+  a.Cu = (uint16_t*)C_up;
+  const int64_t total = (int64_t)a.mtiles * a.ntiles;
+  return swiglu ? gemm_launch<kModeSwiglu>(a, total, (hipStream_t)stream)
+                : gemm_launch<kModeScale>(a, total, (hipStream_t)stream);
+}
+
 }  // namespace
 
 extern "C" int mep_grouped_gemm_nt(const void* A, const void* B, const void* B_up,
                                    const int32_t* cu_seqlens, int G, void* C,
                                    const float* row_scale, int M, int N, int K, int swiglu,
                                    void* stream) {
-  MEP_REQUIRE(A && B && cu_seqlens && C, MEP_ERR_INVALID_ARG);
-  MEP_REQUIRE(M > 0 && N > 0 && K > 0 && G > 0, MEP_ERR_INVALID_ARG);
-  MEP_REQUIRE(!swiglu || (B_up && !row_scale), MEP_ERR_INVALID_ARG);
-  MEP_REQUIRE(M % kBM == 0 && K % kBK == 0 && N % (swiglu ? kBN / 2 : kBN) == 0, MEP_ERR_UNSUPPORTED);
-  MEP_REQUIRE((int64_t)M * (N > K ? N : K) < ((int64_t)1 << 40), MEP_ERR_UNSUPPORTED);
-  MEP_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)B_up % 16 == 0) &&
-                  ((uintptr_t)C % 2 == 0), MEP_ERR_ALIGNMENT);
-  GemmArgs a;
-  a.A = (const uint16_t*)A; a.B = (const uint16_t*)B; a.B2 = (const uint16_t*)B_up;
-  a.cu = cu_seqlens; a.C = (uint16_t*)C; a.scale = row_scale;
-  a.M = M; a.N = N; a.K = K; a.G = G;
-  a.mtiles = M / kBM;
-  a.ntiles = N / (swiglu ? kBN / 2 : kBN);
-  const int64_t total = (int64_t)a.mtiles * a.ntiles;
-  MEP_REQUIRE(total < (1 << 30), MEP_ERR_UNSUPPORTED);
-  const int per_xcd = (int)((total + 7) / 8);
-  const size_t lds = (size_t)kStages * kStage;
-  hipStream_t st = (hipStream_t)stream;
-  {  // 144 KB of dynamic LDS needs the opt-in, once per device
-    static std::atomic<uint64_t> opted{0};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
-    const uint64_t bit = 1ull << (dev & 63);
-    if (!(opted.load(std::memory_order_acquire) & bit)) {
-      e = hipFuncSetAttribute((const void*)grouped_gemm_nt_kernel<true>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e == hipSuccess)
-        e = hipFuncSetAttribute((const void*)grouped_gemm_nt_kernel<false>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return (int)e;
-      opted.fetch_or(bit, std::memory_order_release);
-    }
-  }
-  if (swiglu)
-    hipLaunchKernelGGL(grouped_gemm_nt_kernel<true>, dim3(per_xcd * 8), dim3(kGemmThreads), lds, st, a);
-  else
-    hipLaunchKernelGGL(grouped_gemm_nt_kernel<false>, dim3(per_xcd * 8), dim3(kGemmThreads), lds, st, a);
+  return gemm_nt_forward(A, B, B_up, cu_seqlens, G, C, nullptr, nullptr, row_scale, M, N, K, swiglu, stream);
+}
+
+extern "C" int mep_grouped_swiglu_nt(const void* A, const void* B_gate, const void* B_up,
+                                     const int32_t* cu_seqlens, int G, void* C_act, void* C_gate,
+                                     void* C_up, int M, int N, int K, void* stream) {
+  return gemm_nt_forward(A, B_gate, B_up, cu_seqlens, G, C_act, C_gate, C_up, nullptr, M, N, K, 1, stream);
+}
+
+extern "C" int mep_grouped_gemm_dual_nt(const void* A1, const void* B1, const void* A2, const void* B2,
+                                        const int32_t* cu_seqlens, int G, void* C, int M, int N, int K,
+                                        void* stream) {
+  const int rc = check_nt_shapes(A1, B1, cu_seqlens, C, M, N, K, G, kBN);
+  if (rc != MEP_OK) return rc;
+  MEP_REQUIRE(A2 && B2, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(2 * (int64_t)K < ((int64_t)1 << 30), MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(((uintptr_t)A1 % 16 == 0) && ((uintptr_t)B1 % 16 == 0) && ((uintptr_t)A2 % 16 == 0) &&
+                  ((uintptr_t)B2 % 16 == 0) && ((uintptr_t)C % 2 == 0), MEP_ERR_ALIGNMENT);
+  GemmArgs a = nt_args(A1, B1, B2, cu_seqlens, C, nullptr, M, N, K, G, kBN);
+  a.A2 = (const uint16_t*)A2;
+  return gemm_launch<kModeDual>(a, (int64_t)a.mtiles * a.ntiles, (hipStream_t)stream);
+}
+
+extern "C" int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int32_t* cu_seqlens, int G,
+                                      float* C, int Ma, int Nb, int64_t ld, void* stream) {
+  MEP_REQUIRE(At && Bt && cu_seqlens && C, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(Ma > 0 && Nb > 0 && G > 0 && ld > 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(Ma % kBM == 0 && Nb % kBN == 0 && ld % kBM == 0, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((int64_t)(Ma > Nb ? Ma : Nb) * ld < ((int64_t)1 << 40), MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(((uintptr_t)At % 16 == 0) && ((uintptr_t)Bt % 16 == 0) && ((uintptr_t)C % 4 == 0),
+              MEP_ERR_ALIGNMENT);
+  GemmArgs a{};
+  a.A = (const uint16_t*)At; a.B = (const uint16_t*)Bt; a.cu = cu_seqlens; a.Cf = C;
+  a.M = Ma; a.N = Nb; a.K = 0; a.G = G;
+  a.mtiles = Ma / kBM;
+  a.ntiles = Nb / kBN;
+  a.ld = ld;
+  return gemm_launch<kModeWgrad>(a, (int64_t)a.mtiles * a.ntiles * G, (hipStream_t)stream);
+}
+
+extern "C" int mep_transpose_bf16(const void* src, void* dst, int batch, int rows, int cols, void* stream) {
+  MEP_REQUIRE(src && dst && src != dst, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(batch > 0 && rows > 0 && cols > 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(rows % 64 == 0 && cols % 64 == 0 && batch <= 65535 && rows / 64 <= 65535, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(((uintptr_t)src % 4 == 0) && ((uintptr_t)dst % 4 == 0), MEP_ERR_ALIGNMENT);
+  hipLaunchKernelGGL(transpose16_kernel, dim3(cols / 64, rows / 64, batch), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t*)src, (uint16_t*)dst, rows, cols);
+  return mep_launch_status();
+}
+
+extern "C" int mep_swiglu_bwd(const void* dh, const void* gate_pre, const void* up_pre,
+                              const float* row_scale, const int32_t* cu_seqlens, int G, void* dgate,
+                              void* dup, void* hs, float* dscale, int M, int N, void* stream) {
+  MEP_REQUIRE(dh && gate_pre && up_pre && cu_seqlens && dgate && dup && hs, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(M > 0 && N > 0 && G > 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(N % 8 == 0, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(((uintptr_t)dh % 16 == 0) && ((uintptr_t)gate_pre % 16 == 0) && ((uintptr_t)up_pre % 16 == 0) &&
+                  ((uintptr_t)dgate % 16 == 0) && ((uintptr_t)dup % 16 == 0) && ((uintptr_t)hs % 16 == 0),
+              MEP_ERR_ALIGNMENT);
+  SwigluBwdArgs a;
+  a.dh = (const uint16_t*)dh; a.gate = (const uint16_t*)gate_pre; a.up = (const uint16_t*)up_pre;
+  a.scale = row_scale; a.cu = cu_seqlens;
+  a.dgate = (uint16_t*)dgate; a.dup = (uint16_t*)dup; a.hs = (uint16_t*)hs; a.dscale = dscale;
+  a.M = M; a.N = N; a.G = G;
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3((M + 3) / 4), dim3(256), 0, (hipStream_t)stream, a);
   return mep_launch_status();
 }

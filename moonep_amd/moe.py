@@ -13,14 +13,19 @@ shared ``EmulatedWorld``): every rank dispatches before any rank's experts
 run, every rank's experts finish before any rank combines -- the ordering the
 reference gets from its cross-rank barriers.
 
-The grouped FFN is a plain PyTorch consumer (library GEMMs per group, group
-bounds read on the host) meant for parity tests, not a tuned kernel.
+``grouped_ffn`` is a plain PyTorch consumer (library GEMMs per group, group
+bounds read on the host) meant for parity tests; ``group_expert_ffn_hip`` is the
+same layer stage on the matrix cores, forward and backward: prefetch of the
+compute views, the grouped SwiGLU FFN of every rank, and in backward the grouped
+input / weight gradient GEMMs followed by ``reduce_grad`` in fp32 -- no PyTorch
+GEMM on either pass.
 """
 
 from __future__ import annotations
 
 import torch
 
+from . import ffn
 from .api import Buffer, EmulatedWorld
 from .grad_reduce import launch_grad_reduce
 from .prefetch import launch_prefetch
@@ -141,6 +146,69 @@ class _GroupPrefetch(torch.autograd.Function):
             # the summing half runs here, the slot grads are temporaries nobody reads again
             launch_grad_reduce(grad[r], slots, ctx.etc, rank=r, phase="reduce")
         return None, None, grad
+
+
+class _GroupExpertFFN(torch.autograd.Function):
+    """Rows of every rank through its experts on the matrix cores.
+
+    fp32 master weights in the orientation the kernels read: gate / up
+    [R, epn, H', H], down [R, epn, H, H'].  Forward: bf16 compute views (local
+    experts, then the prefetch slots filled by ``launch_prefetch``), then per rank
+    the fused gate/up GEMM and the down GEMM with the route weight applied.
+    Backward: the grouped gradient GEMMs per rank, then ``launch_grad_reduce``
+    sums every slot's fp32 weight gradient into its owner's."""
+
+    @staticmethod
+    def forward(ctx, group, experts_to_copy, cu_all, rows_all, slots_all, gate_m, up_m, down_m):
+        R, tp = group.R, group.world.token_padding
+        local = [m.detach().to(torch.bfloat16).contiguous() for m in (gate_m, up_m, down_m)]
+        pools = [torch.zeros_like(t) for t in local]
+        for r in range(R):
+            launch_prefetch(tuple(t[r] for t in local), tuple(pools), experts_to_copy, rank=r)
+        views = [torch.cat([l, p], dim=1) for l, p in zip(local, pools)]      # [R, 2*epn, ...]
+        outs, saved = [], []
+        for r in range(R):
+            y, keep = ffn.grouped_ffn_hip_forward(rows_all[r], None if slots_all is None else slots_all[r],
+                                                  cu_all[r], views[0][r], views[1][r], views[2][r],
+                                                  token_padding=tp)
+            outs.append(y)
+            saved.append(keep)
+        ctx.group, ctx.etc, ctx.cu_all, ctx.views, ctx.saved = group, experts_to_copy, cu_all, views, saved
+        ctx.rows_all, ctx.slots_all = rows_all, slots_all
+        return torch.stack(outs)
+
+    @staticmethod
+    def backward(ctx, g_out):
+        group = ctx.group
+        R, epn, tp = group.R, group.epn, group.world.token_padding
+        g_out = g_out.to(torch.bfloat16).contiguous()
+        drows, dslots, dw = [], [], ([], [], [])
+        for r in range(R):
+            res = ffn.grouped_ffn_hip_backward(
+                g_out[r], ctx.rows_all[r], None if ctx.slots_all is None else ctx.slots_all[r],
+                ctx.cu_all[r], ctx.views[0][r], ctx.views[1][r], ctx.views[2][r], ctx.saved[r],
+                token_padding=tp)
+            drows.append(res[0])
+            dslots.append(res[1])
+            for acc, g in zip(dw, res[2:]):
+                acc.append(g)                                                   # [2*epn, ...] fp32
+        grads = []
+        for per_rank in dw:
+            full = torch.stack(per_rank)                                        # [R, 2*epn, ...]
+            own = full[:, :epn].contiguous()
+            slots = full[:, epn:].contiguous()
+            for r in range(R):     # every rank reads before any rank would clear: summing half only
+                launch_grad_reduce(own[r], slots, ctx.etc, rank=r, phase="reduce")
+            grads.append(own)
+        return (None, None, None, torch.stack(drows),
+                None if ctx.slots_all is None else torch.stack(dslots), *grads)
+
+
+def group_expert_ffn_hip(group, experts_to_copy, cu_all, rows_all, slots_all, gate_m, up_m, down_m):
+    """rows [R,NvS,H] bf16, slots [R,NvS] fp32 | None, cu_all [R,2*epn]; fp32 masters gate / up
+    [R,epn,H',H], down [R,epn,H,H'] -> expert outputs [R,NvS,H] bf16.  Differentiable in rows,
+    slots and the three masters; needs token_padding % 128 == 0 and H, H' multiples of 256."""
+    return _GroupExpertFFN.apply(group, experts_to_copy, cu_all, rows_all, slots_all, gate_m, up_m, down_m)
 
 
 def group_dispatch(group, x_all, w_all, topk_all, tpe):

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared():
     text = open(os.path.join(ROOT, "include", "moonep_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(mep_[a-z_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(mep_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_and_binding_list_the_same_symbols():
@@ -99,6 +99,19 @@ def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
     assert lib.mep_grouped_gemm_nt(A, A, None, A, 4, A, None, 128, 128, 64, 1, None) == -1
     assert lib.mep_grouped_gemm_nt(A, A, A, A, 4, A, A, 128, 128, 64, 1, None) == -1
     assert lib.mep_grouped_gemm_nt(A + 8, A, None, A, 4, A, None, 128, 256, 64, 0, None) == -4
+    # the backward pieces
+    assert lib.mep_grouped_swiglu_nt(A, A, None, A, 4, A, A, A, 128, 128, 64, None) == -1   # no up weights
+    assert lib.mep_grouped_swiglu_nt(A, A, A, A, 4, A, A, A, 128, 192, 64, None) == -2      # N % 128 != 0
+    assert lib.mep_grouped_gemm_dual_nt(A, A, None, A, A, 4, A, 128, 256, 64, None) == -1   # second pair missing
+    assert lib.mep_grouped_gemm_dual_nt(A, A, A, A, A, 4, A, 128, 128, 64, None) == -2      # N % 256 != 0
+    assert lib.mep_grouped_gemm_dual_nt(A, A, A + 2, A, A, 4, A, 128, 256, 64, None) == -4
+    assert lib.mep_grouped_gemm_wgrad(A, A, A, 4, A, 100, 256, 1024, None) == -2            # Ma % 128 != 0
+    assert lib.mep_grouped_gemm_wgrad(A, A, A, 4, A, 128, 256, 1000, None) == -2            # ld % 128 != 0
+    assert lib.mep_grouped_gemm_wgrad(A, None, A, 4, A, 128, 256, 1024, None) == -1
+    assert lib.mep_transpose_bf16(A, A, 1, 64, 64, None) == -1                              # in place
+    assert lib.mep_transpose_bf16(A, A + 8192, 1, 64, 96, None) == -2                       # cols % 64 != 0
+    assert lib.mep_swiglu_bwd(A, A, A, None, A, 4, A, A, A, None, 128, 100, None) == -2     # N % 8 != 0
+    assert lib.mep_swiglu_bwd(A, A, None, None, A, 4, A, A, A, None, 128, 128, None) == -1
 
 
 def test_static_scratch_entry_point_rejects_inputs_beyond_its_fixed_size():

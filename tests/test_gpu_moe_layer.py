@@ -131,3 +131,66 @@ def test_moe_layer_forward_on_hip_kernels_only(cuda):
         torch.cuda.synchronize()
         assert torch.equal(captured.view(torch.int16), eager.view(torch.int16))
     group.destroy()
+
+
+_ATEN_GEMMS = {"aten::mm", "aten::bmm", "aten::addmm", "aten::baddbmm", "aten::matmul", "aten::linear",
+               "aten::einsum", "aten::_scaled_mm", "aten::addbmm", "aten::mv", "aten::addmv"}
+
+
+@pytest.mark.parametrize("sigma", [0.0, 2.0])
+def test_moe_layer_forward_and_backward_without_a_torch_gemm(cuda, sigma):
+    """dispatch -> prefetch + grouped FFN on the matrix cores -> combine, forward
+    AND backward through autograd, every GEMM (forward, input gradients, weight
+    gradients) a launch of this library's grouped kernel: the op trace of the
+    whole step holds no aten matrix product.  Values and all gradients against
+    the dense fp32 reference at the bf16 tolerance of the test above."""
+    R, epn, S, K, H, Hp, tp = 4, 2, 40, 3, 256, 256, 128
+    E = R * epn
+    topk = torch.stack([routing.popularity_biased(S, K, E, R, r, sigma, seed=13) for r in range(R)])
+    tpe = routing.tokens_per_expert(topk, E)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(R, S, H, generator=g).to(cuda).requires_grad_()
+    w = torch.softmax(torch.randn(R, S, K, generator=g), -1).to(cuda).requires_grad_()
+    master = [(torch.randn(R, epn, H, Hp, generator=g) * 0.08).to(cuda).requires_grad_() for _ in range(3)]
+    gout = torch.randn(R, S, H, generator=g).to(cuda)
+    topk_d, tpe_d = topk.to(cuda), tpe.to(cuda)
+    # the orientation the kernels read: gate / up [R, epn, H', H], down [R, epn, H, H']
+    gate_m = master[0].detach().transpose(2, 3).contiguous().requires_grad_()
+    up_m = master[1].detach().transpose(2, 3).contiguous().requires_grad_()
+    down_m = master[2].detach().clone().requires_grad_()
+
+    # the op trace sees the autograd thread too: a library product and its two backward products
+    a, b = (torch.randn(8, 8, device=cuda, requires_grad=True) for _ in range(2))
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CPU]) as probe:
+        (a @ b).sum().backward()
+        torch.cuda.synchronize()
+    assert sum(e.count for e in probe.key_averages() if e.key == "aten::mm") == 3
+
+    group = moe.EmulatedGroup(S, H, K, E, R, token_padding=tp)
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CPU]) as prof:
+        rows, slots, cu, plans = moe.group_dispatch(group, x.to(torch.bfloat16), w, topk_d, tpe_d)
+        etc = plans[0].experts_to_copy
+        y = moe.group_expert_ffn_hip(group, etc, cu, rows, slots, gate_m, up_m, down_m)
+        out = moe.group_combine(group, plans, y)
+        (out.float() * gout).sum().backward()
+        torch.cuda.synchronize()
+    ops = {e.key for e in prof.key_averages()}
+    assert "aten::mul" in ops, "the trace must have recorded this step's ops"
+    assert not (ops & _ATEN_GEMMS), f"library matrix products in the step: {sorted(ops & _ATEN_GEMMS)}"
+    if sigma > 0:
+        assert bool((etc >= 0).any()), "the skewed routing must exercise prefetch slots"
+    got = dict(out=out.float().detach(), x=x.grad.clone(), w=w.grad.clone(),
+               m0=gate_m.grad.transpose(2, 3), m1=up_m.grad.transpose(2, 3), m2=down_m.grad)
+    for t in (x, w):
+        t.grad = None
+    ref = _dense_reference(x, w, topk_d, master, epn)
+    (ref * gout).sum().backward()
+    want = dict(out=ref.detach(), x=x.grad, w=w.grad, **{f"m{i}": m.grad for i, m in enumerate(master)})
+    for name in want:
+        a, b = got[name].float(), want[name]
+        scale, err = float(b.abs().max()), float((a - b).abs().max())
+        assert err <= 0.03 * scale + 1e-6, (name, err, scale)
+        cos = float(torch.nn.functional.cosine_similarity(a.flatten(), b.flatten(), dim=0))
+        assert cos > 0.999, (name, cos)
+    assert gate_m.grad.dtype == torch.float32
+    group.destroy()
