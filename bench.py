@@ -82,6 +82,8 @@ def parse():
                     help="no GPU work: turn the counter_collection.csv files of two rocprofv3 --pmc runs of "
                          "`bench.py --profile-kernels` (FETCH_SIZE, WRITE_SIZE) into profiles/traffic.json")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--ffn-only", action="store_true",
+                    help="only the expert FFN section (grouped GEMMs, forward and backward), for profiling it")
     ap.add_argument("--no-limited-cus", action="store_true",
                     help="skip the leg that times the chain on CU-masked streams (under rocprofv3 a process "
                          "that still holds such a stream has crashed in the profiler's exit handlers)")
@@ -631,6 +633,9 @@ def main():
     import torch
 
     torch.cuda.set_device(0)
+    if args.ffn_only:
+        print(json.dumps({"ffn": bench_ffn(args.seed, max(2, args.steps // 4))}))
+        return
     S, H, K, E, R, tp, rank = 4096, 7168, 8, 256, 8, 128, 0
     ch = Chain(S, H, K, E, R, tp, rank, args.maxvio, args.seed)
     if args.profile_kernels:
