@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/moonep_hip.h"
 
 #define MEP_WAVE 64
@@ -25,6 +27,20 @@
 static inline int mep_launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? MEP_OK : (int)e;
+}
+
+// CUs of the current device, asked once per device (-1 when the runtime cannot tell)
+static inline int mep_device_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return -1;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
 }
 
 #if defined(__HIPCC__)

@@ -404,20 +404,6 @@ struct PlanConfig {
   int groups;
 };
 
-// CUs of the current device, asked once per device
-int device_cu_count() {
-  static std::atomic<int> cached[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
-  int n = cached[dev].load(std::memory_order_relaxed);
-  if (n == 0) {
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      return -1;
-    cached[dev].store(n, std::memory_order_relaxed);
-  }
-  return n;
-}
-
 // 0 on success
 int plan_config(int S, int K, int E, int R, PlanConfig* c) {
   c->opt_in = false;
@@ -488,7 +474,7 @@ int plan_launch(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int n
     const size_t want = (a.warm_vecs + per_wg - 1) / per_wg;
     // what the CUs hold beside the planning workgroups at 2048 threads per CU
     // (480 workgroups of 1024 threads on 256 CUs)
-    const int cus = device_cu_count();
+    const int cus = mep_device_cu_count();
     if (cus <= 0) return MEP_ERR_INVALID_ARG;
     const int64_t room = (int64_t)cus * (2048 / c.nt) - (int64_t)c.groups * nranks;
     const size_t cap = room > 0 ? (size_t)room : 0;
