@@ -16,7 +16,8 @@ any cache); its duration inside the timed steps, where the planner launch has
 already pulled the tokens into the last-level cache, is reported beside it.
 
 The same line carries the other configurations: the chain at maxvio 0 .. 4 on
-both shapes (`maxvio_sweep`), prefetch_weight and reduce_grad at
+both shapes (`maxvio_sweep`), the chain at the configuration of the reference's own
+figure (`reference_figure_config`), prefetch_weight and reduce_grad at
 [32, 7168, 2048] per rank for the planner's own slot table and for a table with
 8 slots per rank (`weights`), the expert-side grouped FFN (`ffn`), each with its
 own `roofline` record, and the chain bounded to 32 .. 256 compute units
@@ -712,6 +713,23 @@ def main():
             sweep[f"S{shape[0]}_H{shape[1]}_E{shape[2]}_spread_pct"] = \
                 100.0 * (max(chain_us) - min(chain_us)) / min(chain_us)
         line["maxvio_sweep"] = sweep
+        # the configuration of the reference's own figure (figure/comm_vs_deepep.png: ep = 8,
+        # E = 384, H = 7168, K = 8, S = 8192; H20, read off the chart: planning ~40-50 us,
+        # dispatch + epilogue ~1835-1855 us, combine ~1932-1975 us, both bound by NVLink)
+        c3 = Chain(8192, 7168, K, 384, R, tp, rank, 1.0, args.seed, nsets=3)
+        w3, e3, p3 = measure_chain(c3, sub_steps, 2, kernels=False)
+        b3 = c3.bytes_one_way()
+        line["reference_figure_config"] = {
+            "workload": "S=8192 H=7168 K=8 E=384 R=8 token_padding=128, one rank's share on one GPU (HBM-bound; "
+                        "the reference's figure is NVLink-bound on H20: not the same quantity)",
+            "maxvio": round(c3.maxvio, 3), "chain_us": w3 * 1e3, "GBps": 2 * b3 / w3 / 1e6,
+            "pct_hbm_peak": 2 * b3 / w3 / 1e6 / HBM_PEAK_GBPS * 100.0,
+            "plan_us_in_chain": p3["plan_us_in_chain"], "dispatch_us_in_chain": p3["dispatch_us_in_chain"],
+            "combine_us_in_chain": p3["combine_us_in_chain"],
+            "reference_read_off_its_figure_us": {"planning": "40-50", "dispatch_and_epilogue": "1835-1855",
+                                                 "combine": "1932-1975", "hardware": "H20, 8 GPUs, NVLink"}}
+        c3.destroy()
+        torch.cuda.empty_cache()
         line["weights"] = bench_weights(args.seed, max(5, args.steps // 2), cpu=not args.no_cpu)
         torch.cuda.empty_cache()
         line["ffn"] = bench_ffn(args.seed, max(5, args.steps // 2))

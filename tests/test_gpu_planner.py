@@ -64,6 +64,7 @@ def test_planner_matches_reference_golden(cuda, golden, name):
     (4096, 7168, 8, 256, 8, 0.0),
     (4096, 7168, 8, 256, 8, 4.0),
     (8192, 4096, 8, 128, 8, 2.0),
+    (8192, 7168, 8, 384, 8, 1.0),   # the configuration of the reference's own figure (48 experts per rank)
 ])
 def test_planner_matches_oracle_at_headline_shapes(cuda, S, H, K, E, R, mv):
     topk, _, tpe, real_mv, _ = routing.logit_routing(S, K, E, R, mv, seed=1234, want_weights=False)
