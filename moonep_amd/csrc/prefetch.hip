@@ -254,7 +254,6 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
   t.carve(smem, a.R, a.epn);
   int* occ = smem + slot_table_ints(a.R, a.epn);  // [epn] own slots holding foreign experts, [1] their number
   int64_t* sbase = (int64_t*)(smem + ((slot_table_ints(a.R, a.epn) + a.epn + 2) & ~1));  // [R*epn] byte offset in the pool of list entry i
-  int* sown = (int*)(sbase + a.R * a.epn);                // [R*epn] own slot index of the entry, or -1
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
     const int lo = a.rank * a.epn;
@@ -280,7 +279,6 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
     const int rb = t.list[i];
     const int src = rb / a.epn, b = rb - src * a.epn;
     sbase[i] = ((int64_t)src * a.rank_stride + (int64_t)b * a.elems) * 4;
-    sown[i] = (clear_as_read && src == a.rank) ? b : -1;
   }
   __syncthreads();
   const int64_t work = rt.tiles * n_active;
@@ -325,7 +323,10 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
     const int beg = t.off[le], end = t.off[le + 1];
     auto slot_ptr = [&](int sidx) -> const char* { return (const char*)a.pool + sbase[sidx] + o; };
     // slot sidx belongs to `rank` itself (it then holds one of the rank's own experts)
-    auto own_slot = [&](int sidx) -> int { return sown[sidx]; };
+    auto own_slot = [&](int sidx) -> int {
+      const int b = t.list[sidx] - a.rank * a.epn;
+      return (clear_as_read && (unsigned)b < (unsigned)a.epn) ? b : -1;
+    };
     mep_f4 acc[kVecPerThread];
     if (rt.whole(tile)) {
       // whole tile (workgroup-uniform): unconditional loads; the vectors of the
@@ -459,10 +460,13 @@ extern "C" int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t ra
   MEP_REQUIRE(rank_stride_elems >= elems_per_expert * epn, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(rank_stride_elems % 4 == 0 && (uintptr_t)local_grad % 16 == 0 &&
                   (uintptr_t)reduce_pool % 16 == 0, MEP_ERR_ALIGNMENT);
-  // slot table + own foreign-held slots + per list entry a pool offset and an own-slot index
+  // slot table + own foreign-held slots + a pool offset per list entry
   const size_t lds = slot_table_bytes(R, epn) + ((size_t)epn + 2) * sizeof(int) +
-                     (size_t)R * epn * (sizeof(int64_t) + sizeof(int)) + 8;
-  MEP_REQUIRE(lds <= 64 * 1024, MEP_ERR_UNSUPPORTED);
+                     (size_t)R * epn * sizeof(int64_t) + 8;
+  MEP_REQUIRE(lds <= 150 * 1024, MEP_ERR_UNSUPPORTED);
+  if (lds > 64 * 1024)  // large rank x slot tables: more dynamic LDS than the default limit
+    MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)grad_reduce_kernel,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   ReduceArgs a{local_grad, reduce_pool, rank_stride_elems, elems_per_expert, experts_to_copy,
                rank, epn, R, flags};
   const ReduceTiles rt(elems_per_expert);

@@ -211,6 +211,8 @@ REDUCE_CASES = [
     ("random1", 8, 8, 128, 128, "random", 1, "randn", 16),
     ("random2", 8, 16, 128, 128, "random", 2, "randn", 0),
     ("epn1", 2, 1, 128, 128, "ring", 0, "randn", 0),
+    # 192 KiB per matrix: one 128 KiB block in the spread tile layout, then four tiles of adjacent pieces
+    ("spread_plus_tail", 4, 4, 384, 128, "random", 3, "randn", 16),
 ]
 
 
@@ -263,6 +265,27 @@ def test_grad_reduce_matches_oracle(cuda, case):
     oo.grad_reduce(want, final_pool.clone(), etc, 0)
     torch.cuda.synchronize()
     assert torch.equal(again.cpu().view(torch.int32), want.view(torch.int32))
+
+
+def test_grad_reduce_with_a_table_beyond_64_kb_of_lds(cuda):
+    """R = 128 ranks x 32 slots: the slot table and the per-entry offsets need more dynamic LDS
+    than the default limit; a few ranks against the oracle, bit for bit."""
+    R, epn, H, Hp = 128, 32, 128, 128
+    etc = PLANS["random"](R, epn, 11)
+    g = torch.Generator().manual_seed(77)
+    slots = torch.randn(R, epn, H, Hp, generator=g) * 1e-3 + torch.randn(R, epn, 1, 1, generator=g)
+    pool = slots.to(cuda)
+    etc_dev = etc.to(cuda)
+    for rank in (0, 63, 127):
+        grad = torch.randn(epn, H, Hp, generator=g)
+        want, scratch = grad.clone(), slots.clone()
+        oo.grad_reduce(want, scratch, etc, rank)
+        pool.copy_(slots)
+        got = grad.to(cuda)
+        launch_grad_reduce(got, pool, etc_dev, rank=rank)
+        torch.cuda.synchronize()
+        assert torch.equal(got.cpu().view(torch.int32), want.view(torch.int32)), f"rank {rank} grad"
+        assert torch.equal(pool.cpu().view(torch.int32), scratch.view(torch.int32)), f"rank {rank} clears"
 
 
 def test_grad_reduce_large_offsets(cuda):
