@@ -83,6 +83,27 @@ __global__ __launch_bounds__(WPB * 64) void rows(char* out, const int* row_of, l
   for (int i = 0; i < kPieces; ++i) __builtin_nontemporal_store(z, (u4*)(p + i * 1024));
 }
 
+// persistent form of `rows`: a fixed grid, every wave takes the rows gw, gw + (waves of the grid), ...
+template <int WPB>
+__global__ __launch_bounds__(WPB * 64) void rows_persistent(char* out, const int* row_of, long nrows) {
+  const int lane = threadIdx.x & 63;
+  const long nw = (long)gridDim.x * WPB;
+  for (long gw = (long)blockIdx.x * WPB + (threadIdx.x >> 6); gw < nrows; gw += nw) {
+    const long row = row_of[gw];
+    const u4 z = {1u, 2u, (uint32_t)gw, 4u};
+    char* p = out + row * (kPieces * 1024L) + lane * 16;
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) __builtin_nontemporal_store(z, (u4*)(p + i * 1024));
+  }
+}
+
+// one workgroup of 14 waves per row: every thread stores once, the row's 14 KiB leave together
+__global__ __launch_bounds__(kPieces * 64) void row_burst(char* out, const int* row_of, long nrows) {
+  const long row = row_of[blockIdx.x];
+  const u4 z = {1u, 2u, (uint32_t)blockIdx.x, 4u};
+  __builtin_nontemporal_store(z, (u4*)(out + row * (kPieces * 1024L) + threadIdx.x * 16));
+}
+
 // a WPB-wave workgroup stores WPB adjacent rows starting at start[block]
 template <int WPB>
 __global__ __launch_bounds__(WPB * 64) void runs(char* out, const int* start, long nblocks) {
@@ -204,6 +225,10 @@ int main(int argc, char** argv) {
     report("rows expert segments", time_us([&] { rows<4, 1><<<grid14, 256>>>(out, d_exp, kRows); }, iters));
     report("rows random", time_us([&] { rows<4, 2><<<grid14, 256>>>(out, d_rnd, kRows); }, iters));
     report("rows random, 8 waves/wg", time_us([&] { rows<8, 2><<<(int)(kRows / 8), 512>>>(out, d_rnd, kRows); }, iters));
+    report("rows expert, 256 persistent wgs", time_us([&] { rows_persistent<4><<<256, 256>>>(out, d_exp, kRows); }, iters));
+    report("rows expert, 512 persistent wgs", time_us([&] { rows_persistent<4><<<512, 256>>>(out, d_exp, kRows); }, iters));
+    report("rows expert, 2048 persistent wgs", time_us([&] { rows_persistent<4><<<2048, 256>>>(out, d_exp, kRows); }, iters));
+    report("row_burst expert (14 waves/row)", time_us([&] { row_burst<<<(int)kRows, kPieces * 64>>>(out, d_exp, kRows); }, iters));
     report("runs<16> 224 KiB random", time_us([&] { runs<16><<<(int)(kRows / 16), 1024>>>(out, d_run, kRows / 16); }, iters));
     report("runs_col<16> same runs", time_us([&] { runs_col<16><<<(int)(kRows / 16), 1024>>>(out, d_run, kRows / 16); }, iters));
     report("runs_col<8> 112 KiB random", time_us([&] { runs_col<8><<<(int)(kRows / 8), 512>>>(out, d_run8, kRows / 8); }, iters));
