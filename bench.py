@@ -435,19 +435,38 @@ def bench_weights(seed, steps, cpu=True):
         for b in range(8):
             ring[d, b] = ((d + 1 + b) % R) * epn + (d * 8 + b) % epn
     per = H * Hp
-    local = (torch.randn(epn, H, Hp, device=dev) * 0.02).to(torch.bfloat16)
-    pool = torch.empty(R, epn, H, Hp, dtype=torch.bfloat16, device=dev)
+    # three projections = three different local tensors and three different pools (25 GB), and
+    # every table in three renumbered variants (other local experts, other slots, same counts)
+    # that the timed launches take in turn: no launch finds its experts or its slots in the
+    # 256 MB last-level cache from the projection or the launch before it
+    local = [(torch.randn(epn, H, Hp, device=dev) * 0.02).to(torch.bfloat16) for _ in range(3)]
+    pool = [torch.empty(R, epn, H, Hp, dtype=torch.bfloat16, device=dev) for _ in range(3)]
     res = {"plan_maxvio": mv}
     tables = {"planner": planned, "ring8": ring}
+    NROT = 3
+
+    def renumbered(etc_np, v):
+        """Local expert le -> (le + 11 v) % epn, slot b -> (b + 5 v) % epn."""
+        e = etc_np.copy()
+        m = e >= 0
+        e[m] = (e[m] // epn) * epn + (e[m] % epn + 11 * v) % epn
+        return np.roll(e, 5 * v, axis=1)
+
     stats = {}
     for name, etc_np in tables.items():
         owned = [(int(((etc_np // epn) == r).sum()), r) for r in range(R)]
         n_slots, rank = max(owned)
         active = len({int(e) for e in etc_np.reshape(-1) if e >= 0 and e // epn == rank})
         own_slots = int((etc_np[rank] >= 0).sum())
-        etc = torch.from_numpy(etc_np.astype("int32")).to(dev)
-        stats[name] = (etc, rank, n_slots, active, own_slots)
-        us = time_launches(lambda: launch_prefetch((local,) * 3, (pool,) * 3, etc, rank=rank), steps)
+        variants = [torch.from_numpy(renumbered(etc_np, v).astype("int32")).to(dev) for v in range(NROT)]
+        stats[name] = (variants, rank, n_slots, active, own_slots)
+        k = [0]
+
+        def pf():
+            k[0] += 1
+            launch_prefetch(tuple(local), tuple(pool), variants[k[0] % NROT], rank=rank)
+
+        us = time_launches(pf, steps)
         by = 3 * (active + n_slots) * per * 2   # each owned expert read once, every slot written
         res[name] = {"rank": rank, "slots": n_slots, "active_experts": active,
                      "own_occupied_slots": own_slots, "prefetch_us_3proj": us,
@@ -457,8 +476,14 @@ def bench_weights(seed, steps, cpu=True):
     torch.cuda.empty_cache()
     grad = torch.zeros(epn, H, Hp, dtype=torch.float32, device=dev)
     red = torch.randn(R, epn, H, Hp, dtype=torch.float32, device=dev) * 1e-3
-    for name, (etc, rank, n_slots, active, own_slots) in stats.items():
-        us = time_launches(lambda: launch_grad_reduce(grad, red, etc, rank=rank), steps)
+    for name, (variants, rank, n_slots, active, own_slots) in stats.items():
+        k = [0]
+
+        def gr():
+            k[0] += 1
+            launch_grad_reduce(grad, red, variants[k[0] % NROT], rank=rank)
+
+        us = time_launches(gr, steps)
         by = (n_slots + 2 * active + own_slots) * per * 4   # slots read, grads read+written, clears
         res[name].update({"grad_reduce_us": us, "grad_reduce_bytes": by,
                           "grad_reduce_GBps": by / us / 1e3 if by else 0.0,
