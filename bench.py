@@ -20,8 +20,12 @@ both shapes (`maxvio_sweep`), the chain at the configuration of the reference's 
 figure (`reference_figure_config`), prefetch_weight and reduce_grad at
 [32, 7168, 2048] per rank for the planner's own slot table and for a table with
 8 slots per rank (`weights`), the expert-side grouped FFN (`ffn`), each with its
-own `roofline` record, and the chain bounded to 32 .. 256 compute units
-(`chain_on_limited_cus`).  `--chain-only` skips them.
+own `roofline` record, the chain bounded to 32 .. 256 compute units
+(`chain_on_limited_cus`), and the chain with six rotating sets of destination
+shards beside the same chain on one set (`chain_on_rotating_shards`).  The weight
+leg passes three different tensors for the three projections and rotates
+renumbered variants of each table, so no launch re-reads what the one before
+left in the last-level cache.  `--chain-only` skips them.
 
 The CPU baseline is the scalar C restatement of the same chain
 (oracle/mep_oracle.c), timed on the host next to the GPU.
@@ -319,6 +323,50 @@ def chain_on_limited_cus(ch, steps):
         torch.cuda.current_stream().wait_stream(st)
         out[f"{n}_cus"] = {"plan_us": t[0], "dispatch_us": t[1], "combine_us": t[2],
                            "chain_us": sum(t), "GBps": 2 * by / sum(t) / 1e3}
+    return out
+
+
+def chain_on_rotating_shards(ch, steps, nsets=6):
+    """The chain with the destination shards rotated too: dispatch of step i writes shard set i,
+    combine reads set i+3, written three steps (1.5 GB of rows) earlier, as in a layer whose
+    expert GEMMs run between the two.  Beside it the chain as timed above (one shard set) in
+    the same form.  Equal figures say that the headline does not live on rows that combine
+    finds in the 256 MB last-level cache right after dispatch wrote them."""
+    import torch
+
+    from moonep_amd.combine import launch_combine
+    from moonep_amd.dispatch import launch_dispatch
+
+    ctxs = [ch.ctx]
+    for _ in range(1, nsets):
+        c = dict(ch.ctx)
+        c["hidden_buf"] = torch.zeros_like(ch.ctx["hidden_buf"])
+        c["meta_buf"] = ch.ctx["meta_buf"].clone()
+        ctxs.append(c)
+    ch.plan_fn()
+    for i in range(nsets):
+        launch_dispatch(ctxs[i], ch.hidden[i % len(ch.hidden)], ch.wk, ch.plan, build_dedup_map=False,
+                        write_dups=True)
+    torch.cuda.synchronize()
+    k = [0]
+
+    def chain(shift, rotate):
+        def fn():
+            k[0] += 1
+            i = k[0] % nsets
+            j = i % len(ch.hidden)
+            ch.plan_fn(j)
+            launch_dispatch(ctxs[i if rotate else 0], ch.hidden[j], ch.wk, ch.plan,
+                            build_dedup_map=False, write_dups=True)
+            launch_combine(ctxs[(i + shift) % nsets if rotate else 0], ch.out[j], ch.plan.dst,
+                           ch.out_w, mode="two_level")
+        return fn
+
+    out = {"one_shard_set_us": time_launches(chain(0, False), steps),
+           "rotating_shard_sets_us": time_launches(chain(nsets // 2, True), steps),
+           "shard_sets": nsets, "GB_per_shard_set": ch.ctx["hidden_buf"].numel() * 2 / 1e9}
+    del ctxs
+    torch.cuda.empty_cache()
     return out
 
 
@@ -713,6 +761,8 @@ def main():
     }
     if not (args.chain_only or args.no_limited_cus):
         line["chain_on_limited_cus"] = chain_on_limited_cus(ch, max(5, args.steps // 2))
+    if not args.chain_only:
+        line["chain_on_rotating_shards"] = chain_on_rotating_shards(ch, args.steps)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(ch)
     ch.destroy()
