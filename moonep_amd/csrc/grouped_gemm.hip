@@ -85,19 +85,39 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   // ---- which tile: XCD x (workgroups x, x+8, ...) walks a contiguous range of
-  // tiles; inside a panel of kPanel row tiles the row tile index runs fastest
-  const int per_group = a.mtiles * a.ntiles;
+  // tiles; inside a panel of kPanel row tiles the row tile index runs fastest.
+  // Only the row tiles below the last group's end take part (the row buffer is
+  // sized for the worst case; what lies beyond would leave the last XCDs idle).
+  const int mtiles = MODE == kModeWgrad ? a.mtiles : min(a.mtiles, (a.cu[a.G - 1] + kBM - 1) / kBM);
+  const int per_group = mtiles * a.ntiles;
   const int total = MODE == kModeWgrad ? per_group * a.G : per_group;
   const int per_xcd = (total + 7) >> 3;
-  const int L0 = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (L0 >= total) return;
-  const int tg = MODE == kModeWgrad ? L0 / per_group : 0;  // wgrad: the group is part of the tile index
-  const int L = L0 - tg * per_group;
-  const int panel = L / (kPanel * a.ntiles);
-  const int within = L - panel * (kPanel * a.ntiles);
-  const int ph = min(kPanel, a.mtiles - panel * kPanel);
-  const int nt = within / ph;
-  const int mt = panel * kPanel + (within - nt * ph);
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  if (idx >= per_xcd) return;
+  int tg = 0, mt, nt;
+  if (MODE == kModeWgrad && (mtiles & 7) == 0) {
+    // Weight gradient: every XCD takes an eighth of the row tiles of EVERY group,
+    // group after group.  Groups differ in length (slots are often empty), so
+    // whole groups per XCD would leave the arithmetic to a few of them; this
+    // way all finish together, an XCD's L2 holds its slice of the one operand
+    // and the whole of the other (3 MB at 542 rows), and a group's output is
+    // written by all XCDs at once.
+    const int mpx = mtiles >> 3;
+    tg = idx / (mpx * a.ntiles);
+    const int r = idx - tg * (mpx * a.ntiles);
+    nt = r / mpx;
+    mt = xcd * mpx + (r - nt * mpx);
+  } else {
+    const int L0 = xcd * per_xcd + idx;
+    if (L0 >= total) return;
+    tg = MODE == kModeWgrad ? L0 / per_group : 0;  // wgrad: the group is part of the tile index
+    const int L = L0 - tg * per_group;
+    const int panel = L / (kPanel * a.ntiles);
+    const int within = L - panel * (kPanel * a.ntiles);
+    const int ph = min(kPanel, mtiles - panel * kPanel);
+    nt = within / ph;
+    mt = panel * kPanel + (within - nt * ph);
+  }
   const int m0 = mt * kBM;
   constexpr int kCols = SWIGLU ? kBN / 2 : kBN;  // output columns per tile
   const int n0 = nt * kCols;
@@ -242,7 +262,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
       } else if (MODE == kModeWgrad) {
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          cf[(size_t)m * ldc + n0 + 64 * wn + 32 * j + (lane & 31)] = acc[i][j][v];
+          // streaming stores: 58 MB of output per group passing through L2 as ordinary
+          // writes evicts the operand lines the other tiles of the group still need (9 % slower)
+          __builtin_nontemporal_store(acc[i][j][v], &cf[(size_t)m * ldc + n0 + 64 * wn + 32 * j + (lane & 31)]);
       } else {
         const float sc = a.scale ? a.scale[m] : 1.0f;
 #pragma unroll
