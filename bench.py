@@ -602,24 +602,21 @@ def bench_ffn(seed, steps):
     t3 = time_launches(lambda: torch.matmul(rows[:used], gate[0].t(), out=c), steps)
     peak = 2500.0
     # backward of the same FFN: every GEMM on the grouped kernel; the transposes that give the
-    # operands their other orientation are timed with it
+    # weight gradients' operands their other orientation are timed with it
     del c
     dy = torch.randn(NvS, H, device=dev, generator=g).to(torch.bfloat16)
     _, saved = ffn.grouped_ffn_hip_forward(rows, slots, cu, gate, up, down)
     bw = {}
-    down_t = ffn.transpose_bf16(down)
-    bw["transpose_weights_us"] = 3 * time_launches(lambda: ffn.transpose_bf16(down, down_t), max(2, steps // 2))
-    dh = launch_grouped_gemm_nt(dy, down_t, cu)
-    bw["dh_gemm_us"] = time_launches(lambda: launch_grouped_gemm_nt(dy, down_t, cu, dh), steps)
-    del down_t
+    # the input gradients read the forward pass's weight tensors as they are ([K, N] form)
+    dh = ffn.launch_grouped_gemm_nn(dy, down, cu)
+    bw["dh_gemm_us"] = time_launches(lambda: ffn.launch_grouped_gemm_nn(dy, down, cu, dh), steps)
     sb = ffn.launch_swiglu_bwd(dh, saved[0], saved[1], slots, cu)
     dg, du = sb[0], sb[1]
     bw["swiglu_bwd_us"] = time_launches(lambda: ffn.launch_swiglu_bwd(dh, saved[0], saved[1], slots, cu, sb), steps)
-    gate_n, up_n = ffn.transpose_bf16(gate), ffn.transpose_bf16(up)
-    drows = ffn.launch_grouped_gemm_dual_nt(dg, gate_n, du, up_n, cu)
+    drows = ffn.launch_grouped_gemm_dual_nn(dg, gate, du, up, cu)
     bw["dual_dgrad_gemm_us"] = time_launches(
-        lambda: ffn.launch_grouped_gemm_dual_nt(dg, gate_n, du, up_n, cu, drows), steps)
-    del gate_n, up_n, drows
+        lambda: ffn.launch_grouped_gemm_dual_nn(dg, gate, du, up, cu, drows), steps)
+    del drows
     rows_t, dg_t = ffn.transpose_bf16(rows), ffn.transpose_bf16(dg)
     bw["transpose_activations_us"] = (2 * time_launches(lambda: ffn.transpose_bf16(rows, rows_t), steps)
                                       + 3 * time_launches(lambda: ffn.transpose_bf16(dg, dg_t), steps))
@@ -628,7 +625,7 @@ def bench_ffn(seed, steps):
     del rows_t, dg_t, dg, du, sb, dh, dwg
     gemm_us = bw["dh_gemm_us"] + bw["dual_dgrad_gemm_us"] + 3 * bw["wgrad_gemm_us_each"]
     bw["gemm_TFLOPs"] = 12.0 * used * H * Hp / gemm_us / 1e6
-    bw["total_us"] = gemm_us + bw["swiglu_bwd_us"] + bw["transpose_weights_us"] + bw["transpose_activations_us"]
+    bw["total_us"] = gemm_us + bw["swiglu_bwd_us"] + bw["transpose_activations_us"]
     bw["TFLOPs_with_transposes"] = 12.0 * used * H * Hp / bw["total_us"] / 1e6
     return {
         "rows_in_groups": used, "NvS": NvS, "groups": G, "maxvio": mv, "backward": bw,

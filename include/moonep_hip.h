@@ -258,6 +258,26 @@ int mep_grouped_gemm_dual_nt(const void* A1, const void* B1, const void* A2, con
                              void* stream);
 
 /*
+ * C = bf16(row_scale * A * B[g]) with the weights of a group given as [K, N]
+ * (B [G,K,N] bf16, the output column contiguous): the input gradient of a
+ * projection whose forward pass ran mep_grouped_gemm_nt on the same tensor, with
+ * no transposed copy of the weights.  A [M,K], C [M,N], N % 256 == 0,
+ * K % 64 == 0, M % 128 == 0; row_scale [M] fp32 or NULL.  No counterpart in
+ * the reference.
+ */
+int mep_grouped_gemm_nn(const void* A, const void* B, const int32_t* cu_seqlens, int G, void* C,
+                        const float* row_scale, int M, int N, int K, void* stream);
+
+/*
+ * C = bf16(A1 * B1[g] + A2 * B2[g]), weights [G,K,N], one K loop over both
+ * pairs: the input gradient of the gate/up pair straight from the forward
+ * pass's weight tensors.  No counterpart in the reference.
+ */
+int mep_grouped_gemm_dual_nn(const void* A1, const void* B1, const void* A2, const void* B2,
+                             const int32_t* cu_seqlens, int G, void* C, int M, int N, int K,
+                             void* stream);
+
+/*
  * Weight gradients of the grouped GEMMs from TRANSPOSED activations:
  * C[g] [Ma,Nb] fp32 = At[:, rows of g] * Bt[:, rows of g]^T, At [Ma,ld] and
  * Bt [Nb,ld] bf16 with the rank's rows along the contiguous dimension; the rows

@@ -69,17 +69,41 @@ __device__ __forceinline__ void mep_wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
+typedef short mep_s16x4 __attribute__((ext_vector_type(4)));
+typedef short mep_s16x8 __attribute__((ext_vector_type(8)));
+
+// eight K values of one column from two transposing LDS reads (K rows k .. k+3 and k+4 .. k+7)
+__device__ __forceinline__ mep_bf16x8 mep_tr_pair(const char* lo, const char* hi) {
+  const mep_s16x4 x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) mep_s16x4*)lo);
+  const mep_s16x4 y = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) mep_s16x4*)hi);
+  const mep_s16x8 z = __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(mep_bf16x8, z);
+}
+
 // Producer / consumer waves.  Two producer waves stream the tiles from global
 // memory straight into a ring of three LDS stages (global_load_lds, 16 bytes
 // per lane: no registers, no LDS store instructions), always two K steps
 // ahead; eight consumer waves only read LDS and feed the matrix cores.  One
 // s_barrier per K step hands a filled stage to the consumers and a drained one
 // back to the producers.  A stage row is the bare 128-byte slice; the 16-byte
-// vector q of row r sits at position q ^ (r & 7), so the eight rows a group of
-// eight lanes reads fall into distinct banks.
-template <int MODE>
+// vector q of row r sits at position q ^ (r & 7) ^ ((r >> 3) & 1), so the
+// sixteen rows that sixteen consecutive lanes read cover all 64 banks once (a
+// 16-byte read runs at 256 bytes per clock then; with q ^ (r & 7) alone, which
+// separates only eight rows, at half of that).
+//
+// BKN: the weights are given as [G, K, N] (the output column contiguous), as the
+// backward pass finds them -- dX = dY * W with W stored for Y = X * W^T.  A K
+// step of the weight tile is then 64 rows of 512 bytes in LDS, and a consumer
+// lane gets its eight K values of one column from two transposing LDS reads
+// (ds_read_b64_tr_b16: sixteen lanes read a 4 x 16 block, four rows of 32
+// bytes, and each receives one column of it).  The 16-byte vector v of row k
+// sits at position v ^ 2 (k & 3): the four rows of such a block then cover all
+// banks once.
+template <int MODE, bool BKN = false>
 __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmArgs a) {
   constexpr bool SWIGLU = MODE == kModeSwiglu;
+  static_assert(!BKN || MODE == kModeScale || MODE == kModeDual, "[K, N] weights: plain and dual products only");
+  static_assert(kProducers == 2, "the lane offsets of the pieces assume that a producer wave's pieces share a parity");
   extern __shared__ __attribute__((aligned(1024))) char gsm[];
   __shared__ int s_group;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -154,16 +178,23 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
     const int r = lane >> 3, kv = lane & 7;
     // piece j of a stage: rows 8j .. 8j+7 of the row tile (j < 16), then of the
     // weight tile; this wave moves the pieces j = p, p + kProducers, ...
-    // lane (r, kv) fetches vector kv ^ r of its row into slot (r, kv)
+    // lane (r, kv) fetches vector kv ^ r ^ (piece & 1) of its row into slot (r, kv); this
+    // wave's pieces all have the parity of p
     if (!any) return;
     const size_t goff = MODE == kModeWgrad ? (size_t)kbeg : (size_t)g * a.N * K;
-    const size_t lane_off = (size_t)r * K + ((kv ^ r) * 8);
+    const size_t lane_off = (size_t)r * K + ((kv ^ r ^ (p & 1)) * 8);
     const uint16_t* Ap = a.A + (size_t)m0 * K + lane_off + (MODE == kModeWgrad ? (size_t)kbeg : 0);
-    const uint16_t* Bp0 = a.B + goff + (size_t)n0 * K + lane_off;
+    // [K, N] weights: piece jb holds the K rows 2 jb and 2 jb + 1 of the step; lane (lk, lv)
+    // fetches vector lv ^ 2 (row & 3) of row 2 jb + lk, and (2 jb + lk) & 3 = 2 (p & 1) + lk
+    // because this wave's pieces all have the parity of p
+    const int lk = lane >> 5, lv = lane & 31;
+    const size_t lane_off_kn = (size_t)lk * a.N + (size_t)((lv ^ ((2 * (p & 1) + lk) << 1)) * 8) + n0;
+    const uint16_t* Bp0 = BKN ? a.B + goff + lane_off_kn : a.B + goff + (size_t)n0 * K + lane_off;
     const uint16_t* Bp1 = SWIGLU ? a.B2 + goff + (size_t)n0 * K + lane_off : Bp0 + (size_t)(kBN / 2) * K;
     // dual: the second half of the K loop reads the second pair
     const uint16_t* Aq = MODE == kModeDual ? a.A2 + (size_t)m0 * K + lane_off : Ap;
-    const uint16_t* Bq0 = MODE == kModeDual ? a.B2 + goff + (size_t)n0 * K + lane_off : Bp0;
+    const uint16_t* Bq0 = MODE != kModeDual ? Bp0
+                          : BKN ? a.B2 + goff + lane_off_kn : a.B2 + goff + (size_t)n0 * K + lane_off;
     const uint16_t* Bq1 = Bq0 + (size_t)(kBN / 2) * K;
     auto issue = [&](int k0, int stage) {
       char* base = gsm + stage * kStage;
@@ -177,6 +208,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
         const int j = p + q * kProducers;  // 0 .. 47
         const uint16_t* src;
         if (j < kBM / 8) src = pa + (size_t)(8 * j) * K + k0;
+        else if (BKN) src = pb0 + (size_t)(k0 + 2 * (j - kBM / 8)) * a.N;
         else if (j < kBM / 8 + kBN / 16) src = pb0 + (size_t)(8 * (j - kBM / 8)) * K + k0;
         else src = pb1 + (size_t)(8 * (j - kBM / 8 - kBN / 16)) * K + k0;
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
@@ -214,10 +246,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   const int arow = 64 * wm + (lane & 31);
   const int brow0 = kBM + (SWIGLU ? 32 * wn + (lane & 31) : 64 * wn + (lane & 31));
   const int brow1 = SWIGLU ? brow0 + kBN / 2 : brow0 + 32;
-  const int sw = lane & 7;      // (row & 7) of every operand row of this lane
+  const int sw = (lane & 7) ^ ((lane >> 3) & 1);  // (row & 7) ^ ((row >> 3) & 1) of every operand row of this lane
   const int half = lane >> 5;   // which 8 of the 16 K values of an MFMA step
   const int oa0 = arow * kRowBytes, oa1 = (arow + 32) * kRowBytes;
   const int ob0 = brow0 * kRowBytes, ob1 = brow1 * kRowBytes;
+  // [K, N] weights: lane s of a block of sixteen reads 8 bytes of row 8 half + s / 4 (+ 4 for
+  // the second read, + 16 per MFMA step) at the columns 64 wn + 32 j + 16 (block & 1) + 4 (s & 3)
+  const int ts = lane & 15, tb = (lane >> 4) & 1;
+  const int okn0 = kATile + (8 * half + (ts >> 2)) * (kBN * 2) +
+                   (((8 * wn + 2 * tb + ((ts & 3) >> 1)) ^ ((ts >> 2) << 1)) * 16) + (ts & 1) * 8;
+  const int okn1 = kATile + (8 * half + (ts >> 2)) * (kBN * 2) +
+                   (((8 * wn + 4 + 2 * tb + ((ts & 3) >> 1)) ^ ((ts >> 2) << 1)) * 16) + (ts & 1) * 8;
 
   if (any) {
     __builtin_amdgcn_s_barrier();  // stage 0 is filled
@@ -231,8 +270,15 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
       const int col = ((2 * ks + half) ^ sw) * 16;
       const mep_bf16x8 a0 = *(const mep_bf16x8*)(sb + oa0 + col);
       const mep_bf16x8 a1 = *(const mep_bf16x8*)(sb + oa1 + col);
-      const mep_bf16x8 b0 = *(const mep_bf16x8*)(sb + ob0 + col);
-      const mep_bf16x8 b1 = *(const mep_bf16x8*)(sb + ob1 + col);
+      mep_bf16x8 b0, b1;
+      if (BKN) {
+        const int step = ks * 16 * (kBN * 2);
+        b0 = mep_tr_pair(sb + okn0 + step, sb + okn0 + step + 4 * (kBN * 2));
+        b1 = mep_tr_pair(sb + okn1 + step, sb + okn1 + step + 4 * (kBN * 2));
+      } else {
+        b0 = *(const mep_bf16x8*)(sb + ob0 + col);
+        b1 = *(const mep_bf16x8*)(sb + ob1 + col);
+      }
       acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
       acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
       acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
@@ -370,7 +416,7 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(SwigluBwdArgs a) {
 }
 
 // 144 KB of dynamic LDS needs the opt-in, once per device and kernel
-template <int MODE>
+template <int MODE, bool BKN = false>
 int gemm_launch(const GemmArgs& a, int64_t total, hipStream_t st) {
   MEP_REQUIRE(total > 0 && total < (1 << 30), MEP_ERR_UNSUPPORTED);
   const int per_xcd = (int)((total + 7) / 8);
@@ -381,12 +427,12 @@ int gemm_launch(const GemmArgs& a, int64_t total, hipStream_t st) {
   if (e != hipSuccess) return (int)e;
   const uint64_t bit = 1ull << (dev & 63);
   if (!(opted.load(std::memory_order_acquire) & bit)) {
-    e = hipFuncSetAttribute((const void*)grouped_gemm_nt_kernel<MODE>,
+    e = hipFuncSetAttribute((const void*)grouped_gemm_nt_kernel<MODE, BKN>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
     opted.fetch_or(bit, std::memory_order_release);
   }
-  hipLaunchKernelGGL(grouped_gemm_nt_kernel<MODE>, dim3(per_xcd * 8), dim3(kGemmThreads), lds, st, a);
+  hipLaunchKernelGGL((grouped_gemm_nt_kernel<MODE, BKN>), dim3(per_xcd * 8), dim3(kGemmThreads), lds, st, a);
   return mep_launch_status();
 }
 
@@ -457,6 +503,29 @@ extern "C" int mep_grouped_gemm_dual_nt(const void* A1, const void* B1, const vo
   GemmArgs a = nt_args(A1, B1, B2, cu_seqlens, C, nullptr, M, N, K, G, kBN);
   a.A2 = (const uint16_t*)A2;
   return gemm_launch<kModeDual>(a, (int64_t)a.mtiles * a.ntiles, (hipStream_t)stream);
+}
+
+extern "C" int mep_grouped_gemm_nn(const void* A, const void* B, const int32_t* cu_seqlens, int G, void* C,
+                                   const float* row_scale, int M, int N, int K, void* stream) {
+  const int rc = check_nt_shapes(A, B, cu_seqlens, C, M, N, K, G, kBN);
+  if (rc != MEP_OK) return rc;
+  MEP_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)C % 2 == 0), MEP_ERR_ALIGNMENT);
+  GemmArgs a = nt_args(A, B, nullptr, cu_seqlens, C, row_scale, M, N, K, G, kBN);
+  return gemm_launch<kModeScale, true>(a, (int64_t)a.mtiles * a.ntiles, (hipStream_t)stream);
+}
+
+extern "C" int mep_grouped_gemm_dual_nn(const void* A1, const void* B1, const void* A2, const void* B2,
+                                        const int32_t* cu_seqlens, int G, void* C, int M, int N, int K,
+                                        void* stream) {
+  const int rc = check_nt_shapes(A1, B1, cu_seqlens, C, M, N, K, G, kBN);
+  if (rc != MEP_OK) return rc;
+  MEP_REQUIRE(A2 && B2, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(2 * (int64_t)K < ((int64_t)1 << 30), MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(((uintptr_t)A1 % 16 == 0) && ((uintptr_t)B1 % 16 == 0) && ((uintptr_t)A2 % 16 == 0) &&
+                  ((uintptr_t)B2 % 16 == 0) && ((uintptr_t)C % 2 == 0), MEP_ERR_ALIGNMENT);
+  GemmArgs a = nt_args(A1, B1, B2, cu_seqlens, C, nullptr, M, N, K, G, kBN);
+  a.A2 = (const uint16_t*)A2;
+  return gemm_launch<kModeDual, true>(a, (int64_t)a.mtiles * a.ntiles, (hipStream_t)stream);
 }
 
 extern "C" int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int32_t* cu_seqlens, int G,

@@ -135,6 +135,49 @@ def launch_grouped_gemm_dual_nt(a1, w1, a2, w2, cu_seqlens, out=None, *, token_p
     return out
 
 
+def launch_grouped_gemm_nn(rows, weights_kn, cu_seqlens, out=None, *, row_scale=None, token_padding: int = 128):
+    """``out[m] = rows[m] @ weights_kn[g(m)]`` -> [M, N] bf16; weights_kn [G, K, N] bf16
+    (the tensor a forward ``launch_grouped_gemm_nt`` took as [G, N', K'] = [G, K, N]: its
+    input gradient needs no transposed copy).  Rows at or beyond ``cu_seqlens[-1]`` are
+    not written (zero when ``out`` is allocated here)."""
+    _check_groups(rows, cu_seqlens, token_padding)
+    M, K = rows.shape
+    G = cu_seqlens.numel()
+    _check_weights(weights_kn, G)
+    N = weights_kn.shape[2]
+    _check_weights(weights_kn, G, K, N)
+    if row_scale is not None:
+        assert row_scale.dtype == torch.float32 and row_scale.is_contiguous() and row_scale.numel() == M
+    if out is None:
+        out = torch.zeros(M, N, dtype=torch.bfloat16, device=rows.device)
+    assert out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (M, N)
+    rc = _lib.lib().mep_grouped_gemm_nn(rows.data_ptr(), weights_kn.data_ptr(), cu_seqlens.data_ptr(), G,
+                                        out.data_ptr(), _lib.ptr(row_scale), M, N, K, _lib.current_stream())
+    _lib.check(rc, "mep_grouped_gemm_nn")
+    return out
+
+
+def launch_grouped_gemm_dual_nn(a1, w1_kn, a2, w2_kn, cu_seqlens, out=None, *, token_padding: int = 128):
+    """``a1 @ w1_kn[grp] + a2 @ w2_kn[grp]`` -> [M, N] bf16, weights [G, K, N] (one K loop
+    over both pairs).  Rows at or beyond ``cu_seqlens[-1]`` are not written."""
+    _check_groups(a1, cu_seqlens, token_padding)
+    assert a2.shape == a1.shape and a2.dtype == torch.bfloat16 and a2.is_contiguous()
+    M, K = a1.shape
+    G = cu_seqlens.numel()
+    _check_weights(w1_kn, G)
+    N = w1_kn.shape[2]
+    _check_weights(w1_kn, G, K, N)
+    _check_weights(w2_kn, G, K, N)
+    if out is None:
+        out = torch.zeros(M, N, dtype=torch.bfloat16, device=a1.device)
+    assert out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (M, N)
+    rc = _lib.lib().mep_grouped_gemm_dual_nn(
+        a1.data_ptr(), w1_kn.data_ptr(), a2.data_ptr(), w2_kn.data_ptr(), cu_seqlens.data_ptr(), G,
+        out.data_ptr(), M, N, K, _lib.current_stream())
+    _lib.check(rc, "mep_grouped_gemm_dual_nn")
+    return out
+
+
 def launch_grouped_gemm_wgrad(at, bt, cu_seqlens, out=None, *, token_padding: int = 128):
     """Weight gradients from transposed activations: ``out[g] = at[:, rows of g] @
     bt[:, rows of g].T`` -> fp32 [G, Ma, Nb]; at [Ma, M], bt [Nb, M] bf16 with
@@ -201,16 +244,15 @@ def grouped_ffn_hip_backward(dy, rows, slots, cu_seqlens, gate_t, up_t, down, sa
                              token_padding: int = 128):
     """Backward of ``grouped_ffn_hip``: -> (drows [M,H] bf16, dslots [M] fp32 | None,
     dgate_t, dup_t [G,H',H] fp32, ddown [G,H,H'] fp32).  Every GEMM runs on the
-    matrix cores through the grouped kernel; the operands it needs in the other
-    orientation are transposed first."""
+    matrix cores through the grouped kernel: the input gradients read the weights
+    as they are ([K, N] form), the weight gradients take transposed activations."""
     gp, up = saved
     dy = dy.contiguous()
-    # gradient of the unscaled activation: dy @ W_down, W_down[g] is [H, H'] -> K-contiguous [H', H]
-    dh = launch_grouped_gemm_nt(dy, transpose_bf16(down), cu_seqlens, token_padding=token_padding)
+    # gradient of the unscaled activation: dy @ down[g], down[g] is [H, H'] = [K, N]
+    dh = launch_grouped_gemm_nn(dy, down, cu_seqlens, token_padding=token_padding)
     dg, du, hs, dslots = launch_swiglu_bwd(dh, gp, up, slots, cu_seqlens)
-    # input gradient: dg @ W_gate + du @ W_up, W_gate[g] = gate_t[g].T is [H, H']
-    drows = launch_grouped_gemm_dual_nt(dg, transpose_bf16(gate_t), du, transpose_bf16(up_t), cu_seqlens,
-                                        token_padding=token_padding)
+    # input gradient: dg @ gate_t[g] + du @ up_t[g], both [H', H] = [K, N]
+    drows = launch_grouped_gemm_dual_nn(dg, gate_t, du, up_t, cu_seqlens, token_padding=token_padding)
     rows_t, dy_t = transpose_bf16(rows), transpose_bf16(dy)
     dgate_t = launch_grouped_gemm_wgrad(transpose_bf16(dg), rows_t, cu_seqlens, token_padding=token_padding)
     dup_t = launch_grouped_gemm_wgrad(transpose_bf16(du), rows_t, cu_seqlens, token_padding=token_padding)

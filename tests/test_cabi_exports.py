@@ -105,6 +105,11 @@ def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
     assert lib.mep_grouped_gemm_dual_nt(A, A, None, A, A, 4, A, 128, 256, 64, None) == -1   # second pair missing
     assert lib.mep_grouped_gemm_dual_nt(A, A, A, A, A, 4, A, 128, 128, 64, None) == -2      # N % 256 != 0
     assert lib.mep_grouped_gemm_dual_nt(A, A, A + 2, A, A, 4, A, 128, 256, 64, None) == -4
+    assert lib.mep_grouped_gemm_nn(A, None, A, 4, A, None, 128, 256, 64, None) == -1        # weights missing
+    assert lib.mep_grouped_gemm_nn(A, A, A, 4, A, None, 128, 256, 96, None) == -2           # K % 64 != 0
+    assert lib.mep_grouped_gemm_nn(A, A + 2, A, 4, A, None, 128, 256, 64, None) == -4
+    assert lib.mep_grouped_gemm_dual_nn(A, A, None, A, A, 4, A, 128, 256, 64, None) == -1   # second pair missing
+    assert lib.mep_grouped_gemm_dual_nn(A, A, A, A, A, 4, A, 128, 128, 64, None) == -2      # N % 256 != 0
     assert lib.mep_grouped_gemm_wgrad(A, A, A, 4, A, 100, 256, 1024, None) == -2            # Ma % 128 != 0
     assert lib.mep_grouped_gemm_wgrad(A, A, A, 4, A, 128, 256, 1000, None) == -2            # ld % 128 != 0
     assert lib.mep_grouped_gemm_wgrad(A, None, A, 4, A, 128, 256, 1024, None) == -1

@@ -80,6 +80,38 @@ def test_dual_gemm_sums_both_products(cuda, M, K, N, G, tail):
     assert not got[int(ends[-1]):].any()
 
 
+@pytest.mark.parametrize("M,K,N,G,tail", [(128, 64, 256, 1, 0), (640, 192, 512, 5, 128), (2304, 512, 768, 64, 256)])
+def test_products_with_weights_in_k_by_n_form(cuda, M, K, N, G, tail):
+    """rows @ w[g] with w [G, K, N] (the input gradient's orientation: no transposed copy):
+    against the fp32 product, alone with a row scale and as the sum of two pairs.  The
+    weights carry a different value in every (k, n): a lane that took its K values from the
+    wrong rows or columns of the transposing LDS read would not pass."""
+    g = torch.Generator().manual_seed(M + K + N + 7)
+    a1, a2 = (torch.randn(M, K, generator=g).to(torch.bfloat16) for _ in range(2))
+    w1, w2 = ((torch.randn(G, K, N, generator=g) / K ** 0.5).to(torch.bfloat16) for _ in range(2))
+    scale = torch.rand(M, generator=g) + 0.5
+    ends = _groups(G, M, seed=G * 7 + M, tail=tail)
+    one = ffn.launch_grouped_gemm_nn(a1.to(cuda), w1.to(cuda), ends.to(cuda), row_scale=scale.to(cuda))
+    two = ffn.launch_grouped_gemm_dual_nn(a1.to(cuda), w1.to(cuda), a2.to(cuda), w2.to(cuda), ends.to(cuda))
+    torch.cuda.synchronize()
+    ref1, ref2 = torch.zeros(M, N), torch.zeros(M, N)
+    start = 0
+    for gi, end in enumerate(ends.tolist()):
+        if end > start:
+            p1 = a1[start:end].float() @ w1[gi].float()
+            ref1[start:end] = scale[start:end, None] * p1
+            ref2[start:end] = p1 + a2[start:end].float() @ w2[gi].float()
+        start = max(start, end)
+    _close(one.cpu(), ref1, "nn")
+    _close(two.cpu(), ref2, "dual nn")
+    assert not one[int(ends[-1]):].any() and not two[int(ends[-1]):].any()
+    # the same product through the [N, K] kernel on a transposed copy: same accumulation order
+    # per output element, so the two agree to the bit
+    nt = ffn.launch_grouped_gemm_nt(a1.to(cuda), ffn.transpose_bf16(w1.to(cuda)), ends.to(cuda),
+                                    row_scale=scale.to(cuda))
+    assert torch.equal(nt, one)
+
+
 @pytest.mark.parametrize("M,Ma,Nb,G,tail", [(128, 128, 256, 1, 0), (1024, 256, 512, 6, 256), (2304, 384, 256, 64, 128)])
 def test_weight_gradients_per_group(cuda, M, Ma, Nb, G, tail):
     g = torch.Generator().manual_seed(M + Ma + Nb)
