@@ -25,6 +25,17 @@
 // (one L2) work on the same 8 row tiles and neighbouring weight tiles.
 #include "mep_common.h"
 
+// MEP_GEMM_PROBE (tests/host/gemm_clock_probe only; never defined in the library build):
+// 1 = the kernel as it is, 2 = no global loads (consumers alone), 3 = no LDS reads or MFMAs
+// (producers alone); every tile adds its core clocks and its constant-rate wall ticks to
+// g_gemm_probe, which tells the clock the chip sustains under each of the three.
+#ifndef MEP_GEMM_PROBE
+#define MEP_GEMM_PROBE 0
+#endif
+#if MEP_GEMM_PROBE
+__device__ unsigned long long g_gemm_probe[4];  // core clocks, wall ticks, tiles
+#endif
+
 #include <atomic>
 
 namespace {
@@ -39,7 +50,6 @@ constexpr int kStage = kATile + kBTile;        // 48 KB
 constexpr int kStages = 3;
 constexpr int kConsumers = 8, kProducers = 2;  // waves
 constexpr int kGemmThreads = (kConsumers + kProducers) * 64;
-constexpr int kPanel = 8;  // row tiles that share a sweep over the weight tiles
 // 1 KB pieces (8 rows x 128 bytes) of a stage that one producer wave moves per step
 constexpr int kPiecesPerProducer = (kBM + kBN) / 8 / kProducers;  // 24
 static_assert(2 * kPiecesPerProducer < 64, "two steps of loads must fit the 6-bit load counter");
@@ -105,13 +115,24 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   static_assert(!BKN || MODE == kModeScale || MODE == kModeDual, "[K, N] weights: plain and dual products only");
   static_assert(kProducers == 2, "the lane offsets of the pieces assume that a producer wave's pieces share a parity");
   extern __shared__ __attribute__((aligned(1024))) char gsm[];
-  __shared__ int s_group;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+#if MEP_GEMM_PROBE
+  const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
+#endif
 
-  // ---- which tile: XCD x (workgroups x, x+8, ...) walks a contiguous range of
-  // tiles; inside a panel of kPanel row tiles the row tile index runs fastest.
-  // Only the row tiles below the last group's end take part (the row buffer is
-  // sized for the worst case; what lies beyond would leave the last XCDs idle).
+  // ---- which tile.  XCD x (workgroups x, x+8, ...) walks a contiguous eighth of
+  // the tile list, in launch order, so the tiles that run on an XCD at one time
+  // are neighbours in the list.  Only the row tiles below the last group's end
+  // are listed (the row buffer is sized for the worst case; what lies beyond
+  // would leave the last XCDs idle).
+  //
+  // Row-tiled products: the list goes group by group, inside a group weight tile
+  // by weight tile, the group's row tiles running fastest.  The h row tiles of
+  // a group then read a weight tile at the same time (it leaves HBM once), and
+  // the 32 tiles an XCD runs cover 32 / h weight tiles of that group, so its
+  // rows are fetched ntiles h / 32 times.  (Panels of eight row tiles whatever
+  // the groups were, as before, split most groups over two panels: their
+  // weights came from HBM twice.)
   const int mtiles = MODE == kModeWgrad ? a.mtiles : min(a.mtiles, (a.cu[a.G - 1] + kBM - 1) / kBM);
   const int per_group = mtiles * a.ntiles;
   const int total = MODE == kModeWgrad ? per_group * a.G : per_group;
@@ -119,48 +140,53 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
   if (idx >= per_xcd) return;
   int tg = 0, mt, nt;
-  if (MODE == kModeWgrad && (mtiles & 7) == 0) {
-    // Weight gradient: every XCD takes an eighth of the row tiles of EVERY group,
-    // group after group.  Groups differ in length (slots are often empty), so
-    // whole groups per XCD would leave the arithmetic to a few of them; this
-    // way all finish together, an XCD's L2 holds its slice of the one operand
-    // and the whole of the other (3 MB at 542 rows), and a group's output is
-    // written by all XCDs at once.
-    const int mpx = mtiles >> 3;
-    tg = idx / (mpx * a.ntiles);
-    const int r = idx - tg * (mpx * a.ntiles);
-    nt = r / mpx;
-    mt = xcd * mpx + (r - nt * mpx);
+  if (MODE == kModeWgrad) {
+    if ((mtiles & 7) == 0) {
+      // Weight gradient: every XCD takes an eighth of the row tiles of EVERY group,
+      // group after group.  Groups differ in length (slots are often empty), so
+      // whole groups per XCD would leave the arithmetic to a few of them; this
+      // way all finish together and a group's output is written by all XCDs at once.
+      const int mpx = mtiles >> 3;
+      tg = idx / (mpx * a.ntiles);
+      const int r = idx - tg * (mpx * a.ntiles);
+      nt = r / mpx;
+      mt = xcd * mpx + (r - nt * mpx);
+    } else {
+      const int L0 = xcd * per_xcd + idx;
+      if (L0 >= total) return;
+      tg = L0 / per_group;
+      const int L = L0 - tg * per_group;
+      nt = L / mtiles;
+      mt = L - nt * mtiles;
+    }
   } else {
     const int L0 = xcd * per_xcd + idx;
     if (L0 >= total) return;
-    tg = MODE == kModeWgrad ? L0 / per_group : 0;  // wgrad: the group is part of the tile index
-    const int L = L0 - tg * per_group;
-    const int panel = L / (kPanel * a.ntiles);
-    const int within = L - panel * (kPanel * a.ntiles);
-    const int ph = min(kPanel, mtiles - panel * kPanel);
-    nt = within / ph;
-    mt = panel * kPanel + (within - nt * ph);
+    // the group whose tiles contain list entry L0: the first whose padded end, counted
+    // in tiles, lies beyond it (every wave finds it for itself: 64 groups are one ballot)
+    tg = -1;
+    int beg_tiles = 0, end_tiles = 0;
+    for (int c = 0; c < a.G && tg < 0; c += 64) {
+      const int e = c + lane < a.G ? a.cu[c + lane] / kBM : 0;
+      const uint64_t m = __ballot(c + lane < a.G && e * a.ntiles > L0);
+      if (m) {
+        const int src = __ffsll((unsigned long long)m) - 1;
+        tg = c + src;
+        end_tiles = __shfl(e, src);
+        const int prev = __shfl(e, src > 0 ? src - 1 : 0);
+        beg_tiles = src > 0 ? prev : (c > 0 ? a.cu[c - 1] / kBM : 0);
+      }
+    }
+    if (tg < 0) return;  // cannot happen: L0 < total
+    const int h = end_tiles - beg_tiles;
+    const int local = L0 - beg_tiles * a.ntiles;
+    nt = local / h;
+    mt = beg_tiles + (local - nt * h);
   }
   const int m0 = mt * kBM;
   constexpr int kCols = SWIGLU ? kBN / 2 : kBN;  // output columns per tile
   const int n0 = nt * kCols;
-
-  // ---- group of this row tile: the first whose padded end lies beyond m0
-  if (MODE == kModeWgrad) {
-    if (tid == 0) s_group = tg;
-  } else if (wave == 0) {
-    int g = -1;
-    for (int c = 0; c < a.G && g < 0; c += 64) {
-      const int end = c + lane < a.G ? a.cu[c + lane] : 0;
-      const uint64_t m = __ballot(c + lane < a.G && end > m0);
-      if (m) g = c + __ffsll((unsigned long long)m) - 1;
-    }
-    if (lane == 0) s_group = g;
-  }
-  __syncthreads();
-  const int g = s_group;
-  if (g < 0) return;  // rows past the last group: nothing to compute
+  const int g = tg;
 
   // K steps of this tile and where its K range starts in a row
   int kbeg = 0, KT = a.K / kBK;
@@ -211,9 +237,13 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
         else if (BKN) src = pb0 + (size_t)(k0 + 2 * (j - kBM / 8)) * a.N;
         else if (j < kBM / 8 + kBN / 16) src = pb0 + (size_t)(8 * (j - kBM / 8)) * K + k0;
         else src = pb1 + (size_t)(8 * (j - kBM / 8 - kBN / 16)) * K + k0;
+#if MEP_GEMM_PROBE == 2
+        (void)src; (void)base;
+#else
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                          (__attribute__((address_space(3))) void*)(base + j * 1024),
                                          16, 0, 0);
+#endif
       }
     };
     const int klast = (KT - 1) * kBK;
@@ -267,6 +297,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
     const char* sb = gsm + st * kStage;
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
+#if MEP_GEMM_PROBE == 3
+      continue;
+#endif
       const int col = ((2 * ks + half) ^ sw) * 16;
       const mep_bf16x8 a0 = *(const mep_bf16x8*)(sb + oa0 + col);
       const mep_bf16x8 a1 = *(const mep_bf16x8*)(sb + oa1 + col);
@@ -290,6 +323,13 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   }
 
+#if MEP_GEMM_PROBE
+  if (tid == 0) {
+    atomicAdd(&g_gemm_probe[0], (unsigned long long)(clock64() - probe_c0));
+    atomicAdd(&g_gemm_probe[1], (unsigned long long)(wall_clock64() - probe_w0));
+    atomicAdd(&g_gemm_probe[2], 1ull);
+  }
+#endif
   // ---- epilogue.  acc[i][j][v]: row 64*wm + 32*i + 8*(v/4) + 4*(lane/32) + v%4,
   // column (lane % 32) of the j-th 32-wide block
   const int ldc = a.N;
@@ -477,6 +517,18 @@ int gemm_nt_forward(const void* A, const void* B, const void* B_up, const int32_
 }
 
 }  // namespace
+
+#if MEP_GEMM_PROBE
+extern "C" int mep_gemm_probe_read(unsigned long long* out3, int reset) {
+  hipError_t e = hipMemcpyFromSymbol(out3, HIP_SYMBOL(g_gemm_probe), 3 * sizeof(unsigned long long));
+  if (e != hipSuccess) return (int)e;
+  if (reset) {
+    const unsigned long long z[3] = {0, 0, 0};
+    e = hipMemcpyToSymbol(HIP_SYMBOL(g_gemm_probe), z, sizeof(z));
+  }
+  return (int)e;
+}
+#endif
 
 extern "C" int mep_grouped_gemm_nt(const void* A, const void* B, const void* B_up,
                                    const int32_t* cu_seqlens, int G, void* C,
