@@ -363,6 +363,141 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
 }
 
 // ---------------------------------------------------------------------------
+// Weight gradient on 256 x 256 tiles.  The weight gradient is bound by the
+// lines its tiles load (a K loop of only rows / 64 steps, both operands
+// activations): a 256 x 256 tile needs a third fewer lines per flop than a
+// 128 x 256 one, and both output dimensions are multiples of 256 for the
+// shapes of an expert.  Eight waves of 128 x 64 (128 accumulator registers),
+// all of them load: every wave moves eight of the 64 one-KB pieces of a K step
+// straight into the other of two 64 KB LDS stages before it multiplies the
+// current one; one barrier per step.
+//
+// Tile map: the dimension with more tiles is cut into eight slices, one per
+// XCD (mirrored for odd groups, so that 28 tiles give every XCD 3 + 4), and
+// every XCD takes its slice of every group, two neighbouring groups at a time
+// (pairing every local expert with a slot instead, so that the zeroes of unused
+// slots are written beside the products, was 8 % slower): all XCDs
+// finish together whatever the groups' lengths, and the tiles an XCD runs at
+// one time are one group's slice times the whole other dimension -- each line
+// they load is wanted by 3 to 8 of them.
+// ---------------------------------------------------------------------------
+constexpr int kW2T = 256;                       // tile edge
+constexpr int kW2Stage = 2 * kW2T * kRowBytes;  // 64 KB: 256 rows of each operand
+constexpr int kW2Threads = 512;
+
+struct Wgrad2Map {
+  int sliced, other;  // tiles of the sliced and of the other dimension
+  bool slice_m;       // the sliced dimension is the output row
+  __host__ __device__ int lo(int x) const { return x * sliced / 8; }
+  __host__ __device__ int size(int x) const { return (x + 1) * sliced / 8 - x * sliced / 8; }
+  __host__ __device__ int pair_count(int x) const { return (size(x) + size(7 - x)) * other; }
+};
+
+__global__ __launch_bounds__(kW2Threads, 1) void wgrad256_kernel(GemmArgs a, Wgrad2Map map) {
+  extern __shared__ __attribute__((aligned(1024))) char gsm[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int per_pair = map.pair_count(xcd);
+  if (per_pair == 0 || idx >= per_pair * (a.G >> 1)) return;
+  const int pair = idx / per_pair;
+  int local = idx - pair * per_pair;
+  const int n_even = map.size(xcd) * map.other;
+  int g = 2 * pair, xe = xcd;
+  if (local >= n_even) { local -= n_even; g += 1; xe = 7 - xcd; }
+  const int sz = map.size(xe);
+  const int u = local / sz, sl = map.lo(xe) + (local - u * sz);
+  const int m0 = (map.slice_m ? sl : u) * kW2T, n0 = (map.slice_m ? u : sl) * kW2T;
+  const int kbeg = g > 0 ? a.cu[g - 1] : 0;
+  const int KT = (a.cu[g] - kbeg) / kBK;
+  const size_t ld = (size_t)a.ld;
+
+  // ---- loads: piece j (0 .. 63) is rows 8j .. 8j+7 of the stage (output rows, then output
+  // columns); wave w moves the pieces 8w .. 8w+7; lane (r, kv) fetches vector
+  // kv ^ r ^ (j & 1) of its row into slot (r, kv)
+  const int r = lane >> 3, kv = lane & 7;
+  const uint16_t* src[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const int j = wave * 8 + q;
+    const int row = 8 * j + r;  // 0 .. 511
+    const uint16_t* base = row < kW2T ? a.A + (size_t)(m0 + row) * ld : a.B + (size_t)(n0 + row - kW2T) * ld;
+    src[q] = base + kbeg + ((kv ^ r ^ (q & 1)) * 8);
+  }
+  auto issue = [&](int kt, int stage) {
+    char* base = gsm + stage * kW2Stage + wave * 8 * 1024;
+#pragma unroll
+    for (int q = 0; q < 8; ++q)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + kt * kBK),
+                                       (__attribute__((address_space(3))) void*)(base + q * 1024), 16, 0, 0);
+  };
+
+  float* cf = a.Cf + (size_t)g * a.M * a.N;
+  if (KT == 0) {
+    // a group without rows (an unused slot): its gradient is zero -- whole 1 KB rows of the
+    // tile per wave instruction instead of the accumulators' two 128-byte pieces
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int row = wave; row < kW2T; row += kW2Threads / 64)
+      __builtin_nontemporal_store(zero, (f32x4*)(cf + (size_t)(m0 + row) * a.N + n0) + lane);
+    return;
+  }
+  const int wm = wave & 1, wn = wave >> 1;  // 2 x 4 waves, 128 x 64 each
+  mep_f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+  const int l31 = lane & 31, half = lane >> 5;
+  const int sw = (lane & 7) ^ ((lane >> 3) & 1);
+  const int oa = (128 * wm + l31) * kRowBytes, ob = (kW2T + 64 * wn + l31) * kRowBytes;
+
+  issue(0, 0);
+  mep_wait_vmcnt<0>();
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  for (int kt = 0; kt < KT; ++kt) {
+    const int st = kt & 1;
+    if (kt + 1 < KT) issue(kt + 1, st ^ 1);
+    const char* sb = gsm + st * kW2Stage;
+#pragma unroll
+    for (int ks = 0; ks < kBK / 16; ++ks) {
+      const int col = ((2 * ks + half) ^ sw) * 16;
+      mep_bf16x8 fa[4], fb[2];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) fa[i] = *(const mep_bf16x8*)(sb + oa + i * 32 * kRowBytes + col);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fb[j] = *(const mep_bf16x8*)(sb + ob + j * 32 * kRowBytes + col);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    mep_wait_vmcnt<0>();  // the next stage has landed
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();  // ... for everyone, and everyone is done with this one
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  }
+
+  // ---- epilogue: acc[i][j][v] is row 128 wm + 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,
+  // column 64 wn + 32 j + lane % 32; streaming stores (see the 128 x 256 kernel)
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int m = m0 + 128 * wm + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        __builtin_nontemporal_store(acc[i][j][v], &cf[(size_t)m * a.N + n0 + 64 * wn + 32 * j + l31]);
+    }
+}
+
+
+// ---------------------------------------------------------------------------
 // [batch, rows, cols] -> [batch, cols, rows] of 2-byte elements through a
 // 64 x 64 LDS tile (rows and cols multiples of 64): 128-byte reads and writes.
 // ---------------------------------------------------------------------------
@@ -591,9 +726,33 @@ extern "C" int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int3
   GemmArgs a{};
   a.A = (const uint16_t*)At; a.B = (const uint16_t*)Bt; a.cu = cu_seqlens; a.Cf = C;
   a.M = Ma; a.N = Nb; a.K = 0; a.G = G;
+  a.ld = ld;
+  if (Ma % kW2T == 0 && Nb % kW2T == 0 && G % 2 == 0) {  // the shapes of an expert: 256 x 256 tiles
+    Wgrad2Map map;
+    const int mt = Ma / kW2T, nt = Nb / kW2T;
+    map.slice_m = mt >= nt;
+    map.sliced = map.slice_m ? mt : nt;
+    map.other = map.slice_m ? nt : mt;
+    int per_pair = 0;
+    for (int x = 0; x < 8; ++x) per_pair = per_pair > map.pair_count(x) ? per_pair : map.pair_count(x);
+    const int64_t per_xcd = (int64_t)per_pair * (G / 2);
+    MEP_REQUIRE(per_xcd > 0 && per_xcd < (1 << 27), MEP_ERR_UNSUPPORTED);
+    const size_t lds = 2 * (size_t)kW2Stage;
+    static std::atomic<uint64_t> opted{0};
+    int dev = 0;
+    MEP_RETURN_IF_HIP(hipGetDevice(&dev));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(opted.load(std::memory_order_acquire) & bit)) {
+      MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)wgrad256_kernel,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      opted.fetch_or(bit, std::memory_order_release);
+    }
+    hipLaunchKernelGGL(wgrad256_kernel, dim3((unsigned)(per_xcd * 8)), dim3(kW2Threads), lds, (hipStream_t)stream,
+                       a, map);
+    return mep_launch_status();
+  }
   a.mtiles = Ma / kBM;
   a.ntiles = Nb / kBN;
-  a.ld = ld;
   return gemm_launch<kModeWgrad>(a, (int64_t)a.mtiles * a.ntiles * G, (hipStream_t)stream);
 }
 

@@ -112,7 +112,10 @@ def test_products_with_weights_in_k_by_n_form(cuda, M, K, N, G, tail):
     assert torch.equal(nt, one)
 
 
-@pytest.mark.parametrize("M,Ma,Nb,G,tail", [(128, 128, 256, 1, 0), (1024, 256, 512, 6, 256), (2304, 384, 256, 64, 128)])
+# 128 x 256 tiles (an output dimension that is no multiple of 256, or an odd group count) and
+# 256 x 256 tiles (both are, G even): either output dimension the longer one, 7 tiles over 8 XCDs
+@pytest.mark.parametrize("M,Ma,Nb,G,tail", [(128, 128, 256, 1, 0), (1024, 256, 512, 6, 256), (2304, 384, 256, 64, 128),
+                                            (1152, 512, 1792, 4, 128), (1920, 1792, 256, 8, 0), (768, 256, 256, 3, 0)])
 def test_weight_gradients_per_group(cuda, M, Ma, Nb, G, tail):
     g = torch.Generator().manual_seed(M + Ma + Nb)
     at = torch.randn(Ma, M, generator=g).to(torch.bfloat16)
