@@ -363,6 +363,224 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
 }
 
 // ---------------------------------------------------------------------------
+// Row-tiled products on tiles of 256 (or 128) rows x 256 weight rows.  These
+// kernels are bound by the lines they load, and a 256 x 256 tile needs a third
+// fewer of them per flop than a 128 x 256 one.  Groups end on multiples of 128
+// rows, so a group of h row blocks is covered by h / 2 tiles of 256 rows and,
+// if h is odd, one of 128 (a 256-row tile padded to the next group would load
+// and multiply as much again as it saves).  Eight waves of 128 x 64, all of
+// them load: every wave moves eight of the 64 one-KB pieces of a K step
+// straight into the other of two 64 KB LDS stages before it multiplies the
+// current one; one barrier per step.  A tile of 128 rows loads no rows for the
+// upper four waves' half and those waves only take part in the loads.
+// Tile list as in the kernel above: group by group, weight tile by weight
+// tile, the group's row tiles fastest; XCD x walks the x-th eighth.
+// ---------------------------------------------------------------------------
+constexpr int kT2Rows = 256;
+constexpr int kT2Stage = (kT2Rows + kBN) * kRowBytes;  // 64 KB
+constexpr int kT2Threads = 512;
+constexpr int kT2BOff = kT2Rows * kRowBytes;           // weight rows follow the 256 rows of the row tile
+
+template <int MODE, bool BKN>
+__global__ __launch_bounds__(kT2Threads, 1) void grouped_gemm256_kernel(GemmArgs a) {
+  constexpr bool SWIGLU = MODE == kModeSwiglu;
+  static_assert(MODE == kModeScale || MODE == kModeSwiglu || MODE == kModeDual, "row-tiled products only");
+  static_assert(!BKN || !SWIGLU, "[K, N] weights: plain and dual products only");
+  extern __shared__ __attribute__((aligned(1024))) char gsm[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+#if MEP_GEMM_PROBE
+  const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
+#endif
+
+  // ---- tile list: group g has (h + 1) / 2 row tiles, h = its 128-row blocks
+  int total_rt = 0;
+  for (int c = 0; c < a.G; c += 64) {
+    const int gi = c + lane;
+    const int end = gi < a.G ? a.cu[gi] : 0;
+    const int beg = (gi > 0 && gi < a.G) ? a.cu[gi - 1] : 0;
+    const int t = gi < a.G ? ((end - beg) / kBM + 1) >> 1 : 0;
+    total_rt += __shfl(mep_wave_incl_scan(t), 63);
+  }
+  const int total = total_rt * a.ntiles;
+  const int per_xcd = (total + 7) >> 3;
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  if (idx >= per_xcd) return;
+  const int L0 = xcd * per_xcd + idx;
+  if (L0 >= total) return;
+  int g = -1, m0 = 0, nt = 0;
+  bool tall = true;
+  {
+    int carry = 0;
+    for (int c = 0; c < a.G && g < 0; c += 64) {
+      const int gi = c + lane;
+      const int end = gi < a.G ? a.cu[gi] : 0;
+      const int beg = (gi > 0 && gi < a.G) ? a.cu[gi - 1] : 0;
+      const int t = gi < a.G ? ((end - beg) / kBM + 1) >> 1 : 0;
+      const int incl = carry + mep_wave_incl_scan(t);
+      const uint64_t m = __ballot(gi < a.G && incl * a.ntiles > L0);
+      if (m) {
+        const int src = __ffsll((unsigned long long)m) - 1;
+        g = c + src;
+        const int hs = __shfl(t, src), first = __shfl(incl - t, src);
+        const int gbeg = __shfl(beg, src), gend = __shfl(end, src);
+        const int local = L0 - first * a.ntiles;
+        nt = local / hs;
+        m0 = gbeg + (local - nt * hs) * kT2Rows;
+        tall = m0 + kT2Rows <= gend;
+      }
+      carry = __shfl(incl, 63);
+    }
+  }
+  if (g < 0) return;  // cannot happen: L0 < total
+  constexpr int kCols = SWIGLU ? kBN / 2 : kBN;  // output columns per tile
+  const int n0 = nt * kCols;
+  const int KT1 = a.K / kBK;
+  const int KT = MODE == kModeDual ? 2 * KT1 : KT1;
+  const size_t K = (size_t)a.ld;
+
+  // ---- loads.  Piece j (0 .. 63) is rows 8j .. 8j+7 of the stage (the row tile, then the
+  // weight tile); wave w moves the pieces 8w .. 8w+7, so the waves 0-3 load rows and the waves
+  // 4-7 weights.  Lane (r, kv) fetches vector kv ^ r ^ (j & 1) of its row into slot (r, kv).
+  // [K, N] weights: weight piece jb holds the K rows 2 jb and 2 jb + 1 of the step, lane
+  // (lk, lv) fetches vector lv ^ 2 ((2 jb + lk) & 3) of its row.
+  const bool loads_rows = wave < 4;
+  const bool idle_loader = !tall && (wave == 2 || wave == 3);  // rows 128 .. 255 of a 128-row tile
+  const uint16_t* src[8];
+  size_t kstep;         // elements per K step
+  ptrdiff_t delta = 0;  // distance to the second pair (dual), elements
+  {
+    const int r = lane >> 3, kv = lane & 7, lk = lane >> 5, lv = lane & 31;
+    const size_t goff = (size_t)g * a.N * K;
+    kstep = (BKN && !loads_rows) ? (size_t)kBK * a.N : (size_t)kBK;
+    if (MODE == kModeDual) delta = loads_rows ? a.A2 - a.A : a.B2 - a.B;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int j = wave * 8 + q;
+      if (loads_rows) {
+        const int row = 8 * j + r;
+        src[q] = a.A + (size_t)(m0 + (idle_loader ? 0 : row)) * K + ((kv ^ r ^ (q & 1)) * 8);
+      } else if (BKN) {
+        const int jb = j - 32;
+        src[q] = a.B + goff + (size_t)(2 * jb + lk) * a.N + n0 + ((lv ^ ((2 * (q & 1) + lk) << 1)) * 8);
+      } else {
+        const int rb = 8 * (j - 32) + r;  // 0 .. 255
+        const uint16_t* base = (SWIGLU && rb >= kBN / 2) ? a.B2 : a.B;
+        const int nrow = SWIGLU ? n0 + (rb & (kBN / 2 - 1)) : n0 + rb;
+        src[q] = base + goff + (size_t)nrow * K + ((kv ^ r ^ (q & 1)) * 8);
+      }
+    }
+  }
+  auto issue = [&](int kt, int stage) {
+    if (idle_loader) return;
+    ptrdiff_t off = (ptrdiff_t)((size_t)kt * kstep);
+    if (MODE == kModeDual && kt >= KT1) off = (ptrdiff_t)((size_t)(kt - KT1) * kstep) + delta;
+    char* base = gsm + stage * kT2Stage + wave * 8 * 1024;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+#if MEP_GEMM_PROBE == 2
+      (void)base; (void)off;
+#else
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + off),
+                                       (__attribute__((address_space(3))) void*)(base + q * 1024), 16, 0, 0);
+#endif
+    }
+  };
+
+  // ---- consumers: 2 x 4 waves, 128 x 64 each
+  const int wm = wave & 1, wn = wave >> 1;
+  const bool works = tall || wm == 0;
+  mep_f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+  const int l31 = lane & 31, half = lane >> 5;
+  const int sw = (lane & 7) ^ ((lane >> 3) & 1);
+  const int oa = (128 * wm + l31) * kRowBytes;
+  const int ob0 = kT2BOff + (SWIGLU ? 32 * wn + l31 : 64 * wn + l31) * kRowBytes;
+  const int ob1 = ob0 + (SWIGLU ? kBN / 2 : 32) * kRowBytes;
+  const int ts = lane & 15, tb = (lane >> 4) & 1;
+  const int okn0 = kT2BOff + (8 * half + (ts >> 2)) * (kBN * 2) +
+                   (((8 * wn + 2 * tb + ((ts & 3) >> 1)) ^ ((ts >> 2) << 1)) * 16) + (ts & 1) * 8;
+  const int okn1 = kT2BOff + (8 * half + (ts >> 2)) * (kBN * 2) +
+                   (((8 * wn + 4 + 2 * tb + ((ts & 3) >> 1)) ^ ((ts >> 2) << 1)) * 16) + (ts & 1) * 8;
+
+  issue(0, 0);
+  mep_wait_vmcnt<0>();
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  for (int kt = 0; kt < KT; ++kt) {
+    const int st = kt & 1;
+    if (kt + 1 < KT) issue(kt + 1, st ^ 1);
+    const char* sb = gsm + st * kT2Stage;
+    if (works) {
+#pragma unroll
+      for (int ks = 0; ks < kBK / 16; ++ks) {
+#if MEP_GEMM_PROBE == 3
+        continue;
+#endif
+        const int col = ((2 * ks + half) ^ sw) * 16;
+        mep_bf16x8 fa[4], fb[2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[i] = *(const mep_bf16x8*)(sb + oa + i * 32 * kRowBytes + col);
+        if (BKN) {
+          const int step = ks * 16 * (kBN * 2);
+          fb[0] = mep_tr_pair(sb + okn0 + step, sb + okn0 + step + 4 * (kBN * 2));
+          fb[1] = mep_tr_pair(sb + okn1 + step, sb + okn1 + step + 4 * (kBN * 2));
+        } else {
+          fb[0] = *(const mep_bf16x8*)(sb + ob0 + col);
+          fb[1] = *(const mep_bf16x8*)(sb + ob1 + col);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+    }
+    mep_wait_vmcnt<0>();  // the next stage has landed
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();  // ... for everyone, and everyone is done with this one
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  }
+#if MEP_GEMM_PROBE
+  if (tid == 0) {
+    atomicAdd(&g_gemm_probe[0], (unsigned long long)(clock64() - probe_c0));
+    atomicAdd(&g_gemm_probe[1], (unsigned long long)(wall_clock64() - probe_w0));
+    atomicAdd(&g_gemm_probe[2], 1ull);
+  }
+#endif
+  if (!works) return;
+
+  // ---- epilogue.  acc[i][j][v]: row 128 wm + 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,
+  // column lane % 32 of the j-th 32-wide block
+  const int ldc = a.N;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int m = m0 + 128 * wm + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+      if (SWIGLU) {
+        const int n = n0 + 32 * wn + l31;
+        const float res = mep_silu(acc[i][0][v]) * acc[i][1][v];
+        a.C[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(res);
+        if (a.Cg) a.Cg[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(acc[i][0][v]);
+        if (a.Cu) a.Cu[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(acc[i][1][v]);
+      } else {
+        const float sc = (MODE == kModeScale && a.scale) ? a.scale[m] : 1.0f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int n = n0 + 64 * wn + 32 * j + l31;
+          a.C[(size_t)m * ldc + n] = (uint16_t)mep_f32_to_bf16_bits(sc * acc[i][j][v]);
+        }
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Weight gradient on 256 x 256 tiles.  The weight gradient is bound by the
 // lines its tiles load (a K loop of only rows / 64 steps, both operands
 // activations): a 256 x 256 tile needs a third fewer lines per flop than a
@@ -590,6 +808,28 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(SwigluBwdArgs a) {
   }
 }
 
+// launch of the 256-row-tile kernel: the grid covers the most row tiles the groups can need
+// ((M / 128 + G) / 2, when every group has an odd number of 128-row blocks)
+template <int MODE, bool BKN>
+int gemm256_launch(const GemmArgs& a, hipStream_t st) {
+  const int64_t row_tiles = ((int64_t)a.M / kBM + a.G + 1) / 2;
+  const int64_t total = row_tiles * a.ntiles;
+  MEP_REQUIRE(total > 0 && total < (1 << 30), MEP_ERR_UNSUPPORTED);
+  const int per_xcd = (int)((total + 7) / 8);
+  const size_t lds = 2 * (size_t)kT2Stage;
+  static std::atomic<uint64_t> opted{0};
+  int dev = 0;
+  MEP_RETURN_IF_HIP(hipGetDevice(&dev));
+  const uint64_t bit = 1ull << (dev & 63);
+  if (!(opted.load(std::memory_order_acquire) & bit)) {
+    MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)grouped_gemm256_kernel<MODE, BKN>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    opted.fetch_or(bit, std::memory_order_release);
+  }
+  hipLaunchKernelGGL((grouped_gemm256_kernel<MODE, BKN>), dim3(per_xcd * 8), dim3(kT2Threads), lds, st, a);
+  return mep_launch_status();
+}
+
 // 144 KB of dynamic LDS needs the opt-in, once per device and kernel
 template <int MODE, bool BKN = false>
 int gemm_launch(const GemmArgs& a, int64_t total, hipStream_t st) {
@@ -632,6 +872,21 @@ GemmArgs nt_args(const void* A, const void* B, const void* B2, const int32_t* cu
   return a;
 }
 
+// Which row tiling: 256-row tiles load a third fewer lines per flop, but with two 64 KB
+// stages their loads drain at every K step, and there are half as many tiles to spread over
+// the CUs.  Measured at 34 688 rows, H = 7168, H' = 2048: 5-8 % faster where a launch has at
+// least eight of them per CU (SwiGLU, down, the dual input gradient), 12 % slower at five
+// (dy * down, 2048 output columns).
+// MEP_GEMM_ROW_TILE=128 or 256 in the environment forces one (tests run both on small shapes).
+static bool use_256_row_tiles(const GemmArgs& a) {
+  if (const char* e = getenv("MEP_GEMM_ROW_TILE")) {
+    if (e[0] == '2') return true;
+    if (e[0] == '1') return false;
+  }
+  const int cus = mep_device_cu_count();
+  return (int64_t)(a.M / kT2Rows) * a.ntiles >= 8 * (int64_t)(cus > 0 ? cus : 256);
+}
+
 int gemm_nt_forward(const void* A, const void* B, const void* B_up, const int32_t* cu, int G, void* C,
                     void* C_gate, void* C_up, const float* row_scale, int M, int N, int K, int swiglu,
                     void* stream) {
@@ -647,6 +902,9 @@ int gemm_nt_forward(const void* A, const void* B, const void* B_up, const int32_
   a.Cg = (uint16_t*)C_gate;
   a.Cu = (uint16_t*)C_up;
   const int64_t total = (int64_t)a.mtiles * a.ntiles;
+  if (use_256_row_tiles(a))
+    return swiglu ? gemm256_launch<kModeSwiglu, false>(a, (hipStream_t)stream)
+                  : gemm256_launch<kModeScale, false>(a, (hipStream_t)stream);
   return swiglu ? gemm_launch<kModeSwiglu>(a, total, (hipStream_t)stream)
                 : gemm_launch<kModeScale>(a, total, (hipStream_t)stream);
 }
@@ -689,6 +947,7 @@ extern "C" int mep_grouped_gemm_dual_nt(const void* A1, const void* B1, const vo
                   ((uintptr_t)B2 % 16 == 0) && ((uintptr_t)C % 2 == 0), MEP_ERR_ALIGNMENT);
   GemmArgs a = nt_args(A1, B1, B2, cu_seqlens, C, nullptr, M, N, K, G, kBN);
   a.A2 = (const uint16_t*)A2;
+  if (use_256_row_tiles(a)) return gemm256_launch<kModeDual, false>(a, (hipStream_t)stream);
   return gemm_launch<kModeDual>(a, (int64_t)a.mtiles * a.ntiles, (hipStream_t)stream);
 }
 
@@ -698,6 +957,7 @@ extern "C" int mep_grouped_gemm_nn(const void* A, const void* B, const int32_t* 
   if (rc != MEP_OK) return rc;
   MEP_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)C % 2 == 0), MEP_ERR_ALIGNMENT);
   GemmArgs a = nt_args(A, B, nullptr, cu_seqlens, C, row_scale, M, N, K, G, kBN);
+  if (use_256_row_tiles(a)) return gemm256_launch<kModeScale, true>(a, (hipStream_t)stream);
   return gemm_launch<kModeScale, true>(a, (int64_t)a.mtiles * a.ntiles, (hipStream_t)stream);
 }
 
@@ -712,6 +972,7 @@ extern "C" int mep_grouped_gemm_dual_nn(const void* A1, const void* B1, const vo
                   ((uintptr_t)B2 % 16 == 0) && ((uintptr_t)C % 2 == 0), MEP_ERR_ALIGNMENT);
   GemmArgs a = nt_args(A1, B1, B2, cu_seqlens, C, nullptr, M, N, K, G, kBN);
   a.A2 = (const uint16_t*)A2;
+  if (use_256_row_tiles(a)) return gemm256_launch<kModeDual, true>(a, (hipStream_t)stream);
   return gemm_launch<kModeDual, true>(a, (int64_t)a.mtiles * a.ntiles, (hipStream_t)stream);
 }
 

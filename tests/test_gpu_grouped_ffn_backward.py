@@ -16,6 +16,14 @@ from moonep_amd import ffn
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["128", "256"])
+def row_tile(request, monkeypatch):
+    """Every test runs on both row tilings of the grouped kernel (the library picks by shape;
+    the small shapes here would only ever see one of them)."""
+    monkeypatch.setenv("MEP_GEMM_ROW_TILE", request.param)
+    return request.param
+
+
 def _groups(G, M, seed, tail):
     g = torch.Generator().manual_seed(seed)
     tiles = (M - tail) // 128
