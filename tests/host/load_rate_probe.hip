@@ -28,19 +28,21 @@ __device__ __forceinline__ void wait_vmcnt() {
 
 // share != 0: the workgroups of one XCD read the same region (it stays in their L2);
 // share == 0: every workgroup streams a region of its own from HBM.
-template <int WAVES, int PER, bool TO_LDS>
+template <int WAVES, int PER, bool TO_LDS, bool HALF = false>
 __global__ __launch_bounds__(WAVES * 64, 1) void rate(const char* src, size_t region, size_t stride,
                                                       int rounds, uint32_t* sink, int share) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane >> 3, kv = lane & 7;
+  // HALF: one instruction = 16 rows x 64 bytes (a K step of 32 bf16: half a line per row; the other
+  // half is asked for a whole sweep over the row blocks later)
+  const int r = HALF ? lane >> 2 : lane >> 3, kv = HALF ? lane & 3 : lane & 7;
   const size_t base = (share ? (size_t)(blockIdx.x & 7) : (size_t)blockIdx.x) * region;
   const char* p0 = src + base + (size_t)r * stride + kv * 16;
   // a wave walks the row blocks wave, wave + WAVES, ... of the region, then the next 128-byte column
-  const int nblk = (int)(region / stride / 8), ncol = (int)(stride / 128);
+  const int nblk = (int)(region / stride / (HALF ? 16 : 8)), ncol = (int)(stride / (HALF ? 64 : 128));
   int rb = wave % nblk, col = 0;
   auto next = [&]() {
-    const char* p = p0 + (size_t)rb * 8 * stride + (size_t)col * 128;
+    const char* p = p0 + (size_t)rb * (HALF ? 16 : 8) * stride + (size_t)col * (HALF ? 64 : 128);
     rb += WAVES;
     if (rb >= nblk) {
       rb -= nblk;
@@ -94,9 +96,10 @@ int main() {
   hipEvent_t e0, e1;
   CK(hipEventCreate(&e0));
   CK(hipEventCreate(&e1));
-#define RUN(W, PER, TO_LDS, SHARE, NAME)                                                               \
+#define RUN(W, PER, TO_LDS, SHARE, NAME) RUNH(W, PER, TO_LDS, false, SHARE, NAME)
+#define RUNH(W, PER, TO_LDS, HALF, SHARE, NAME)                                                             \
   {                                                                                                    \
-    auto k = rate<W, PER, TO_LDS>;                                                                     \
+    auto k = rate<W, PER, TO_LDS, HALF>;                                                                  \
     CK(hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024));   \
     const int rounds = (SHARE) ? 32000 / (W * PER) + 8 : (int)(region_hbm / (W * PER * 1024));         \
     const size_t region = (SHARE) ? region_l2 : region_hbm;                                            \
@@ -127,6 +130,8 @@ int main() {
   RUN(4, 12, true, 0, "to LDS, from HBM")
   RUN(8, 8, true, 0, "to LDS, from HBM")
   RUN(16, 4, true, 0, "to LDS, from HBM")
+  RUNH(8, 8, true, true, 1, "to LDS, 64 B, L2 hits")
+  RUNH(8, 8, true, true, 0, "to LDS, 64 B, from HBM")
   RUN(8, 8, false, 0, "to registers, from HBM")
   RUN(16, 8, false, 0, "to registers, from HBM")
   CK(hipFree(buf));
