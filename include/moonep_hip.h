@@ -290,6 +290,16 @@ int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int32_t* cu_seq
                            float* C, int Ma, int Nb, int64_t ld, void* stream);
 
 /*
+ * The same weight gradients from the activations as the passes hold them:
+ * C[g] [Ma,Nb] fp32 = X1[rows of g]^T * X2[rows of g], X1 [rows,Ma] and X2
+ * [rows,Nb] bf16 row-major -- no transposed copies.  Ma % 256 == 0,
+ * Nb % 256 == 0, G even (MEP_ERR_UNSUPPORTED otherwise: transpose and call
+ * mep_grouped_gemm_wgrad).  No counterpart in the reference.
+ */
+int mep_grouped_gemm_wgrad_tn(const void* X1, const void* X2, const int32_t* cu_seqlens, int G,
+                              float* C, int Ma, int Nb, int64_t rows, void* stream);
+
+/*
  * [batch, rows, cols] -> [batch, cols, rows] of bf16 (any 2-byte element);
  * rows % 64 == 0, cols % 64 == 0, src != dst.  Feeds mep_grouped_gemm_wgrad
  * and the backward GEMMs, which want the other operand orientation.

@@ -615,6 +615,10 @@ struct Wgrad2Map {
   __host__ __device__ int pair_count(int x) const { return (size(x) + size(7 - x)) * other; }
 };
 
+// TN: the operands are given as the forward and backward passes hold them, X1 [rows, Ma] and
+// X2 [rows, Nb] (a K step is then 64 rows of 512 bytes of each in LDS, read with the transposing
+// LDS loads of the [K, N] weight form above); otherwise as transposed copies [Ma, rows], [Nb, rows].
+template <bool TN>
 __global__ __launch_bounds__(kW2Threads, 1) void wgrad256_kernel(GemmArgs a, Wgrad2Map map) {
   extern __shared__ __attribute__((aligned(1024))) char gsm[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -635,21 +639,38 @@ __global__ __launch_bounds__(kW2Threads, 1) void wgrad256_kernel(GemmArgs a, Wgr
 
   // ---- loads: piece j (0 .. 63) is rows 8j .. 8j+7 of the stage (output rows, then output
   // columns); wave w moves the pieces 8w .. 8w+7; lane (r, kv) fetches vector
-  // kv ^ r ^ (j & 1) of its row into slot (r, kv)
+  // kv ^ r ^ (j & 1) of its row into slot (r, kv).  TN: piece jp of an operand's half of the
+  // stage is the K rows 2 jp and 2 jp + 1 of the step (256 columns = 512 bytes each); lane
+  // (lk, lv) fetches vector lv ^ 2 ((2 jp + lk) & 3) of its row.
   const int r = lane >> 3, kv = lane & 7;
   const uint16_t* src[8];
+  size_t kstep;  // elements per K step
+  if (TN) {
+    const int lk = lane >> 5, lv = lane & 31;
+    const bool first = wave < 4;  // the waves 0-3 load X1, the waves 4-7 X2
+    const size_t pitch = first ? (size_t)a.M : (size_t)a.N;
+    const uint16_t* base = (first ? a.A + m0 : a.B + n0) + (size_t)kbeg * pitch;
+    kstep = (size_t)kBK * pitch;
 #pragma unroll
-  for (int q = 0; q < 8; ++q) {
-    const int j = wave * 8 + q;
-    const int row = 8 * j + r;  // 0 .. 511
-    const uint16_t* base = row < kW2T ? a.A + (size_t)(m0 + row) * ld : a.B + (size_t)(n0 + row - kW2T) * ld;
-    src[q] = base + kbeg + ((kv ^ r ^ (q & 1)) * 8);
+    for (int q = 0; q < 8; ++q) {
+      const int jp = (wave & 3) * 8 + q;
+      src[q] = base + (size_t)(2 * jp + lk) * pitch + ((lv ^ ((2 * (q & 1) + lk) << 1)) * 8);
+    }
+  } else {
+    kstep = kBK;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int j = wave * 8 + q;
+      const int row = 8 * j + r;  // 0 .. 511
+      const uint16_t* base = row < kW2T ? a.A + (size_t)(m0 + row) * ld : a.B + (size_t)(n0 + row - kW2T) * ld;
+      src[q] = base + kbeg + ((kv ^ r ^ (q & 1)) * 8);
+    }
   }
   auto issue = [&](int kt, int stage) {
     char* base = gsm + stage * kW2Stage + wave * 8 * 1024;
 #pragma unroll
     for (int q = 0; q < 8; ++q)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + kt * kBK),
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + (size_t)kt * kstep),
                                        (__attribute__((address_space(3))) void*)(base + q * 1024), 16, 0, 0);
   };
 
@@ -675,6 +696,12 @@ __global__ __launch_bounds__(kW2Threads, 1) void wgrad256_kernel(GemmArgs a, Wgr
   const int l31 = lane & 31, half = lane >> 5;
   const int sw = (lane & 7) ^ ((lane >> 3) & 1);
   const int oa = (128 * wm + l31) * kRowBytes, ob = (kW2T + 64 * wn + l31) * kRowBytes;
+  // TN: lane s of a block of sixteen reads 8 bytes of K row 8 half + s / 4 (+ 4 for the second
+  // read, + 16 per MFMA step) at the columns c + 16 (block & 1) + 4 (s & 3) of a 32-column block
+  // that starts at column c of its operand's half of the stage
+  const int ts = lane & 15, tb = (lane >> 4) & 1;
+  const int otn = (8 * half + (ts >> 2)) * (kW2T * 2) + (ts & 1) * 8;
+  const int vtn = 2 * tb + ((ts & 3) >> 1), xtn = (ts >> 2) << 1;
 
   issue(0, 0);
   mep_wait_vmcnt<0>();
@@ -689,10 +716,26 @@ __global__ __launch_bounds__(kW2Threads, 1) void wgrad256_kernel(GemmArgs a, Wgr
     for (int ks = 0; ks < kBK / 16; ++ks) {
       const int col = ((2 * ks + half) ^ sw) * 16;
       mep_bf16x8 fa[4], fb[2];
+      if (TN) {
+        // block i (32 columns = 4 vectors) moves the vector index by 4 i; the XOR with xtn
+        // (0, 2, 4 or 6) touches the bits 1 and 2 only, so 4 i is added before it
+        const int step = ks * 16 * (kW2T * 2);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) fa[i] = *(const mep_bf16x8*)(sb + oa + i * 32 * kRowBytes + col);
+        for (int i = 0; i < 4; ++i) {
+          const int o = otn + step + (((16 * wm + 4 * i + vtn) ^ xtn) * 16);
+          fa[i] = mep_tr_pair(sb + o, sb + o + 4 * (kW2T * 2));
+        }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) fb[j] = *(const mep_bf16x8*)(sb + ob + j * 32 * kRowBytes + col);
+        for (int j = 0; j < 2; ++j) {
+          const int o = kW2T * kRowBytes + otn + step + (((8 * wn + 4 * j + vtn) ^ xtn) * 16);
+          fb[j] = mep_tr_pair(sb + o, sb + o + 4 * (kW2T * 2));
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[i] = *(const mep_bf16x8*)(sb + oa + i * 32 * kRowBytes + col);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fb[j] = *(const mep_bf16x8*)(sb + ob + j * 32 * kRowBytes + col);
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -855,6 +898,32 @@ int gemm_launch(const GemmArgs& a, int64_t total, hipStream_t st) {
   return mep_launch_status();
 }
 
+// launch of the 256 x 256 weight gradient (a.M, a.N multiples of 256, a.G even)
+template <bool TN>
+int wgrad256_launch(const GemmArgs& a, hipStream_t st) {
+  Wgrad2Map map;
+  const int mt = a.M / kW2T, nt = a.N / kW2T;
+  map.slice_m = mt >= nt;
+  map.sliced = map.slice_m ? mt : nt;
+  map.other = map.slice_m ? nt : mt;
+  int per_pair = 0;
+  for (int x = 0; x < 8; ++x) per_pair = per_pair > map.pair_count(x) ? per_pair : map.pair_count(x);
+  const int64_t per_xcd = (int64_t)per_pair * (a.G / 2);
+  MEP_REQUIRE(per_xcd > 0 && per_xcd < (1 << 27), MEP_ERR_UNSUPPORTED);
+  const size_t lds = 2 * (size_t)kW2Stage;
+  static std::atomic<uint64_t> opted{0};
+  int dev = 0;
+  MEP_RETURN_IF_HIP(hipGetDevice(&dev));
+  const uint64_t bit = 1ull << (dev & 63);
+  if (!(opted.load(std::memory_order_acquire) & bit)) {
+    MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)wgrad256_kernel<TN>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    opted.fetch_or(bit, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(wgrad256_kernel<TN>, dim3((unsigned)(per_xcd * 8)), dim3(kW2Threads), lds, st, a, map);
+  return mep_launch_status();
+}
+
 int check_nt_shapes(const void* A, const void* B, const int32_t* cu, const void* C, int M, int N, int K,
                     int G, int cols_per_tile) {
   MEP_REQUIRE(A && B && cu && C, MEP_ERR_INVALID_ARG);
@@ -992,33 +1061,26 @@ extern "C" int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int3
   a.A = (const uint16_t*)At; a.B = (const uint16_t*)Bt; a.cu = cu_seqlens; a.Cf = C;
   a.M = Ma; a.N = Nb; a.K = 0; a.G = G;
   a.ld = ld;
-  if (Ma % kW2T == 0 && Nb % kW2T == 0 && G % 2 == 0) {  // the shapes of an expert: 256 x 256 tiles
-    Wgrad2Map map;
-    const int mt = Ma / kW2T, nt = Nb / kW2T;
-    map.slice_m = mt >= nt;
-    map.sliced = map.slice_m ? mt : nt;
-    map.other = map.slice_m ? nt : mt;
-    int per_pair = 0;
-    for (int x = 0; x < 8; ++x) per_pair = per_pair > map.pair_count(x) ? per_pair : map.pair_count(x);
-    const int64_t per_xcd = (int64_t)per_pair * (G / 2);
-    MEP_REQUIRE(per_xcd > 0 && per_xcd < (1 << 27), MEP_ERR_UNSUPPORTED);
-    const size_t lds = 2 * (size_t)kW2Stage;
-    static std::atomic<uint64_t> opted{0};
-    int dev = 0;
-    MEP_RETURN_IF_HIP(hipGetDevice(&dev));
-    const uint64_t bit = 1ull << (dev & 63);
-    if (!(opted.load(std::memory_order_acquire) & bit)) {
-      MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)wgrad256_kernel,
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      opted.fetch_or(bit, std::memory_order_release);
-    }
-    hipLaunchKernelGGL(wgrad256_kernel, dim3((unsigned)(per_xcd * 8)), dim3(kW2Threads), lds, (hipStream_t)stream,
-                       a, map);
-    return mep_launch_status();
-  }
+  if (Ma % kW2T == 0 && Nb % kW2T == 0 && G % 2 == 0 && (uintptr_t)C % 16 == 0)  // an expert's shapes: 256 x 256 tiles
+    return wgrad256_launch<false>(a, (hipStream_t)stream);
   a.mtiles = Ma / kBM;
   a.ntiles = Nb / kBN;
   return gemm_launch<kModeWgrad>(a, (int64_t)a.mtiles * a.ntiles * G, (hipStream_t)stream);
+}
+
+extern "C" int mep_grouped_gemm_wgrad_tn(const void* X1, const void* X2, const int32_t* cu_seqlens, int G,
+                                         float* C, int Ma, int Nb, int64_t rows, void* stream) {
+  MEP_REQUIRE(X1 && X2 && cu_seqlens && C, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(Ma > 0 && Nb > 0 && G > 0 && rows > 0, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(Ma % kW2T == 0 && Nb % kW2T == 0 && G % 2 == 0 && rows % kBM == 0, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((int64_t)(Ma > Nb ? Ma : Nb) * rows < ((int64_t)1 << 40), MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE(((uintptr_t)X1 % 16 == 0) && ((uintptr_t)X2 % 16 == 0) && ((uintptr_t)C % 16 == 0),
+              MEP_ERR_ALIGNMENT);
+  GemmArgs a{};
+  a.A = (const uint16_t*)X1; a.B = (const uint16_t*)X2; a.cu = cu_seqlens; a.Cf = C;
+  a.M = Ma; a.N = Nb; a.K = 0; a.G = G;
+  a.ld = rows;
+  return wgrad256_launch<true>(a, (hipStream_t)stream);
 }
 
 extern "C" int mep_transpose_bf16(const void* src, void* dst, int batch, int rows, int cols, void* stream) {

@@ -196,6 +196,29 @@ def launch_grouped_gemm_wgrad(at, bt, cu_seqlens, out=None, *, token_padding: in
     return out
 
 
+def wgrad_tn_supported(Ma: int, Nb: int, G: int) -> bool:
+    """Shapes `launch_grouped_gemm_wgrad_tn` takes (an expert's: multiples of 256, G even)."""
+    return Ma % 256 == 0 and Nb % 256 == 0 and G % 2 == 0
+
+
+def launch_grouped_gemm_wgrad_tn(x1, x2, cu_seqlens, out=None, *, token_padding: int = 128):
+    """Weight gradients from the activations as they are: ``out[g] = x1[rows of g].T @
+    x2[rows of g]`` -> fp32 [G, Ma, Nb]; x1 [M, Ma], x2 [M, Nb] bf16, no transposed copies."""
+    _check_groups(x1, cu_seqlens, token_padding)
+    assert x2.dtype == torch.bfloat16 and x2.is_contiguous() and x2.dim() == 2 and x2.shape[0] == x1.shape[0]
+    M, Ma = x1.shape
+    Nb = x2.shape[1]
+    G = cu_seqlens.numel()
+    assert wgrad_tn_supported(Ma, Nb, G), f"needs Ma, Nb multiples of 256 and an even G, got {Ma}, {Nb}, {G}"
+    if out is None:
+        out = torch.empty(G, Ma, Nb, dtype=torch.float32, device=x1.device)
+    assert out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (G, Ma, Nb)
+    rc = _lib.lib().mep_grouped_gemm_wgrad_tn(x1.data_ptr(), x2.data_ptr(), cu_seqlens.data_ptr(), G,
+                                              out.data_ptr(), Ma, Nb, M, _lib.current_stream())
+    _lib.check(rc, "mep_grouped_gemm_wgrad_tn")
+    return out
+
+
 def transpose_bf16(t, out=None):
     """[..., rows, cols] -> [..., cols, rows], contiguous (rows, cols multiples of 64)."""
     assert t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous() and t.dim() >= 2
@@ -253,6 +276,12 @@ def grouped_ffn_hip_backward(dy, rows, slots, cu_seqlens, gate_t, up_t, down, sa
     dg, du, hs, dslots = launch_swiglu_bwd(dh, gp, up, slots, cu_seqlens)
     # input gradient: dg @ gate_t[g] + du @ up_t[g], both [H', H] = [K, N]
     drows = launch_grouped_gemm_dual_nn(dg, gate_t, du, up_t, cu_seqlens, token_padding=token_padding)
+    if wgrad_tn_supported(dg.shape[1], rows.shape[1], cu_seqlens.numel()):
+        # an expert's shapes: the weight gradients read the activations as they are
+        dgate_t = launch_grouped_gemm_wgrad_tn(dg, rows, cu_seqlens, token_padding=token_padding)
+        dup_t = launch_grouped_gemm_wgrad_tn(du, rows, cu_seqlens, token_padding=token_padding)
+        ddown = launch_grouped_gemm_wgrad_tn(dy, hs, cu_seqlens, token_padding=token_padding)
+        return drows, dslots, dgate_t, dup_t, ddown
     rows_t, dy_t = transpose_bf16(rows), transpose_bf16(dy)
     dgate_t = launch_grouped_gemm_wgrad(transpose_bf16(dg), rows_t, cu_seqlens, token_padding=token_padding)
     dup_t = launch_grouped_gemm_wgrad(transpose_bf16(du), rows_t, cu_seqlens, token_padding=token_padding)

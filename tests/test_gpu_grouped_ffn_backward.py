@@ -130,6 +130,12 @@ def test_weight_gradients_per_group(cuda, M, Ma, Nb, G, tail):
     bt = torch.randn(Nb, M, generator=g).to(torch.bfloat16)
     ends = _groups(G, M, seed=G * 5 + M, tail=tail)
     got = ffn.launch_grouped_gemm_wgrad(at.to(cuda), bt.to(cuda), ends.to(cuda))
+    if ffn.wgrad_tn_supported(Ma, Nb, G):
+        # the same products from the untransposed activations: same K order per output element,
+        # so the same bits
+        tn = ffn.launch_grouped_gemm_wgrad_tn(at.t().contiguous().to(cuda), bt.t().contiguous().to(cuda),
+                                              ends.to(cuda))
+        assert torch.equal(tn, got)
     torch.cuda.synchronize()
     got = got.cpu()
     start, empty = 0, 0
