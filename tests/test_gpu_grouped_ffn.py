@@ -59,7 +59,8 @@ def _close(got, ref, what):
     (512, 256, 256, 4, 0),
     (1024, 448, 768, 6, 256),      # K = 7 steps, unused rows at the end, empty groups likely
     (2304, 1024, 512, 64, 128),    # more groups than row tiles
-    (1152, 2048, 1280, 3, 0),      # tile counts that are not multiples of the panel size
+    (1152, 2048, 1280, 3, 0),      # tile counts that are no multiples of eight
+    (6400, 128, 256, 96, 256),     # more than 64 groups (E = 384 on 8 ranks): the group search takes two rounds
 ])
 def test_grouped_gemm_matches_fp32_reference(cuda, M, K, N, G, tail):
     g = torch.Generator().manual_seed(M + K + N)

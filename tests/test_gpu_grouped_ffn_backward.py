@@ -88,7 +88,8 @@ def test_dual_gemm_sums_both_products(cuda, M, K, N, G, tail):
     assert not got[int(ends[-1]):].any()
 
 
-@pytest.mark.parametrize("M,K,N,G,tail", [(128, 64, 256, 1, 0), (640, 192, 512, 5, 128), (2304, 512, 768, 64, 256)])
+@pytest.mark.parametrize("M,K,N,G,tail", [(128, 64, 256, 1, 0), (640, 192, 512, 5, 128), (2304, 512, 768, 64, 256),
+                                          (6400, 128, 256, 96, 128)])
 def test_products_with_weights_in_k_by_n_form(cuda, M, K, N, G, tail):
     """rows @ w[g] with w [G, K, N] (the input gradient's orientation: no transposed copy):
     against the fp32 product, alone with a row scale and as the sum of two pairs.  The
