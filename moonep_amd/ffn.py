@@ -12,11 +12,14 @@ capturable in a HIP graph); ``grouped_ffn_hip`` chains the fused gate/up
 Weights are K-contiguous: gate and up views are ``[2*epn, H', H]``, the down
 view is ``[2*epn, H, H']`` -- the layout ``x @ W.T`` reads directly.
 
-The backward pass runs on the same kernel: ``grouped_ffn_hip_backward`` needs
-the operands in the other orientation (weights for the input gradients,
-activations for the weight gradients), which ``transpose_bf16`` makes; the
-weight gradients come out in fp32 ``[2*epn, ...]`` -- local experts first, then
-the slots -- which is what ``launch_grad_reduce`` sums.
+The backward pass runs on the same kernels with the operands as the passes hold
+them: the input gradients read the forward weights in ``[K, N]`` form
+(``launch_grouped_gemm_nn``, ``launch_grouped_gemm_dual_nn``), the weight
+gradients the activations as ``[rows, features]``
+(``launch_grouped_gemm_wgrad_tn``; shapes it does not take go through
+``transpose_bf16`` and ``launch_grouped_gemm_wgrad``).  The weight gradients
+come out in fp32 ``[2*epn, ...]`` -- local experts first, then the slots --
+which is what ``launch_grad_reduce`` sums.
 """
 
 from __future__ import annotations
@@ -267,8 +270,9 @@ def grouped_ffn_hip_backward(dy, rows, slots, cu_seqlens, gate_t, up_t, down, sa
                              token_padding: int = 128):
     """Backward of ``grouped_ffn_hip``: -> (drows [M,H] bf16, dslots [M] fp32 | None,
     dgate_t, dup_t [G,H',H] fp32, ddown [G,H,H'] fp32).  Every GEMM runs on the
-    matrix cores through the grouped kernel: the input gradients read the weights
-    as they are ([K, N] form), the weight gradients take transposed activations."""
+    matrix cores through the grouped kernels: the input gradients read the weights
+    as they are ([K, N] form), the weight gradients the activations as they are
+    (transposed copies only for shapes the untransposed form does not take)."""
     gp, up = saved
     dy = dy.contiguous()
     # gradient of the unscaled activation: dy @ down[g], down[g] is [H, H'] = [K, N]
