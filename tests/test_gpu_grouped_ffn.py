@@ -87,6 +87,23 @@ def test_grouped_gemm_matches_fp32_reference(cuda, M, K, N, G, tail):
     assert (out.cpu()[last:] == 3.0).all()
 
 
+def test_no_rows_at_all(cuda):
+    """Every group empty (a rank that received nothing): the products write nothing, the
+    weight gradients are zero."""
+    from moonep_amd import ffn
+    M, K, N, G = 512, 128, 256, 4
+    rows = torch.randn(M, K).to(torch.bfloat16).to(cuda)
+    w = torch.randn(G, N, K).to(torch.bfloat16).to(cuda)
+    ends = torch.zeros(G, dtype=torch.int32, device=cuda)
+    out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=cuda)
+    launch_grouped_gemm_nt(rows, w, ends, out)
+    ffn.launch_grouped_gemm_nn(rows, w.transpose(1, 2).contiguous(), ends, out)
+    assert bool((out == 7.0).all())
+    wide = torch.cat([rows, rows], 1)   # [M, 256]
+    dw = ffn.launch_grouped_gemm_wgrad_tn(wide, wide, ends)
+    assert not dw.any()
+
+
 def test_grouped_ffn_matches_the_torch_consumer(cuda):
     """Same contract as moonep_amd.moe.grouped_ffn (library GEMMs per group)."""
     from moonep_amd.moe import grouped_ffn
