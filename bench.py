@@ -95,6 +95,9 @@ def parse():
     ap.add_argument("--profile-kernels", action="store_true",
                     help="for rocprofv3: a few plain launches of each kernel and of a 512 MiB "
                          "torch copy (the known-size kernel counters are scaled by); no JSON")
+    ap.add_argument("--profile-weights", action="store_true",
+                    help="for rocprofv3 --pmc: three rounds of a 512 MiB copy, prefetch_weight and reduce_grad "
+                         "on the table with 8 slots per rank, then exit")
     ap.add_argument("--maxvio", type=float, default=1.0)
     ap.add_argument("--seed", type=int, default=2024)
     return ap.parse_args()
@@ -368,6 +371,45 @@ def chain_on_rotating_shards(ch, steps, nsets=6):
     del ctxs
     torch.cuda.empty_cache()
     return out
+
+
+def profile_weights():
+    """Launches for a counter run: a 512 MiB copy (the scale of FETCH_SIZE / WRITE_SIZE), then
+    prefetch_weight (3 projections) and reduce_grad (one projection) at [32, 7168, 2048], R = 8,
+    every rank hosting 8 remote experts, three times on three renumbered tables."""
+    import numpy as np
+    import torch
+
+    from moonep_amd.grad_reduce import launch_grad_reduce
+    from moonep_amd.prefetch import launch_prefetch
+
+    E, R, H, Hp = 256, 8, 7168, 2048
+    epn, rank = E // R, 7
+    dev = torch.device("cuda", 0)
+    ring = -np.ones((R, epn), dtype=np.int64)
+    for d in range(R):
+        for b in range(8):
+            ring[d, b] = ((d + 1 + b) % R) * epn + (d * 8 + b) % epn
+    local = [(torch.randn(epn, H, Hp, device=dev) * 0.02).to(torch.bfloat16) for _ in range(3)]
+    pool = [torch.empty(R, epn, H, Hp, dtype=torch.bfloat16, device=dev) for _ in range(3)]
+    grad = torch.zeros(epn, H, Hp, dtype=torch.float32, device=dev)
+    red = torch.randn(R, epn, H, Hp, dtype=torch.float32, device=dev) * 1e-3
+    src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).view(torch.float32)
+    dst = torch.empty_like(src)
+    for v in range(3):
+        e = ring.copy()
+        m = e >= 0
+        e[m] = (e[m] // epn) * epn + (e[m] % epn + 11 * v) % epn
+        etc = torch.from_numpy(np.roll(e, 5 * v, axis=1).astype("int32")).to(dev)
+        dst.copy_(src)
+        launch_prefetch(tuple(local), tuple(pool), etc, rank=rank)
+        launch_grad_reduce(grad, red, etc, rank=rank)
+        torch.cuda.synchronize()
+    per = H * Hp
+    print(json.dumps({"profile_weights": {"launches_each": 3, "prefetch_bytes": 3 * 16 * per * 2,
+                                          "prefetch_read_bytes": 3 * 8 * per * 2,
+                                          "grad_reduce_bytes": 32 * per * 4,
+                                          "grad_reduce_read_bytes": 16 * per * 4}}), file=sys.stderr)
 
 
 def cpu_baseline(ch, budget_s=10.0):
@@ -701,6 +743,9 @@ def main():
     import torch
 
     torch.cuda.set_device(0)
+    if args.profile_weights:
+        profile_weights()
+        return
     if args.ffn_only:
         print(json.dumps({"ffn": bench_ffn(args.seed, max(2, args.steps // 4))}))
         return
