@@ -50,6 +50,7 @@ constexpr int kStage = kATile + kBTile;        // 48 KB
 constexpr int kStages = 3;
 constexpr int kConsumers = 8, kProducers = 2;  // waves
 constexpr int kGemmThreads = (kConsumers + kProducers) * 64;
+constexpr int kPanel = 8;  // row tiles of a long group that share a sweep over the weight tiles
 // 1 KB pieces (8 rows x 128 bytes) of a stage that one producer wave moves per step
 constexpr int kPiecesPerProducer = (kBM + kBN) / 8 / kProducers;  // 24
 static_assert(2 * kPiecesPerProducer < 64, "two steps of loads must fit the 6-bit load counter");
@@ -67,6 +68,7 @@ struct GemmArgs {
   uint16_t* Cu;        // swiglu: up pre-activation [M,N] or null
   float* Cf;           // wgrad: [G,M,N] fp32
   int64_t ld;          // row stride of A and B in elements (K, or the row count for wgrad)
+  int panel;           // row tiles of a long group that share a sweep over the weight tiles
 };
 
 enum { kModeScale = 0, kModeSwiglu = 1, kModeDual = 2, kModeWgrad = 3 };
@@ -178,10 +180,15 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
       }
     }
     if (tg < 0) return;  // cannot happen: L0 < total
+    // a long group goes in panels of a.panel row tiles (its weights are then read once per
+    // panel, its rows once per 32 / a.panel weight tiles)
     const int h = end_tiles - beg_tiles;
     const int local = L0 - beg_tiles * a.ntiles;
-    nt = local / h;
-    mt = beg_tiles + (local - nt * h);
+    const int panel = local / (a.panel * a.ntiles);
+    const int within = local - panel * (a.panel * a.ntiles);
+    const int ph = min(a.panel, h - panel * a.panel);
+    nt = within / ph;
+    mt = beg_tiles + panel * a.panel + (within - nt * ph);
   }
   const int m0 = mt * kBM;
   constexpr int kCols = SWIGLU ? kBN / 2 : kBN;  // output columns per tile
@@ -383,6 +390,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
 constexpr int kT2Rows = 256;
 constexpr int kT2Stage = (kT2Rows + kBN) * kRowBytes;  // 64 KB
 constexpr int kT2Threads = 512;
+constexpr int kT2Panel = 8;  // row tiles of a long group that share a sweep over the weight tiles (4: 2-3 % slower at 3-6 per group)
 constexpr int kT2BOff = kT2Rows * kRowBytes;           // weight rows follow the 256 rows of the row tile
 
 template <int MODE, bool BKN>
@@ -428,8 +436,12 @@ __global__ __launch_bounds__(kT2Threads, 1) void grouped_gemm256_kernel(GemmArgs
         const int hs = __shfl(t, src), first = __shfl(incl - t, src);
         const int gbeg = __shfl(beg, src), gend = __shfl(end, src);
         const int local = L0 - first * a.ntiles;
-        nt = local / hs;
-        m0 = gbeg + (local - nt * hs) * kT2Rows;
+        // a long group goes in panels of a.panel row tiles
+        const int panel = local / (a.panel * a.ntiles);
+        const int within = local - panel * (a.panel * a.ntiles);
+        const int ph = min(a.panel, hs - panel * a.panel);
+        nt = within / ph;
+        m0 = gbeg + (panel * a.panel + (within - nt * ph)) * kT2Rows;
         tall = m0 + kT2Rows <= gend;
       }
       carry = __shfl(incl, 63);
@@ -858,7 +870,9 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(SwigluBwdArgs a) {
 // launch of the 256-row-tile kernel: the grid covers the most row tiles the groups can need
 // ((M / 128 + G) / 2, when every group has an odd number of 128-row blocks)
 template <int MODE, bool BKN>
-int gemm256_launch(const GemmArgs& a, hipStream_t st) {
+int gemm256_launch(const GemmArgs& a0, hipStream_t st) {
+  GemmArgs a = a0;
+  a.panel = kT2Panel;
   const int64_t row_tiles = ((int64_t)a.M / kBM + a.G + 1) / 2;
   const int64_t total = row_tiles * a.ntiles;
   MEP_REQUIRE(total > 0 && total < (1 << 30), MEP_ERR_UNSUPPORTED);
@@ -879,7 +893,9 @@ int gemm256_launch(const GemmArgs& a, hipStream_t st) {
 
 // 144 KB of dynamic LDS needs the opt-in, once per device and kernel
 template <int MODE, bool BKN = false>
-int gemm_launch(const GemmArgs& a, int64_t total, hipStream_t st) {
+int gemm_launch(const GemmArgs& a0, int64_t total, hipStream_t st) {
+  GemmArgs a = a0;
+  a.panel = kPanel;
   MEP_REQUIRE(total > 0 && total < (1 << 30), MEP_ERR_UNSUPPORTED);
   const int per_xcd = (int)((total + 7) / 8);
   const size_t lds = (size_t)kStages * kStage;
