@@ -659,8 +659,13 @@ def bench_ffn(seed, steps):
         lambda: ffn.launch_grouped_gemm_dual_nn(dg, gate, du, up, cu, drows), steps)
     del drows
     # the weight gradients read the activations as they are (an expert's shapes: no transposes)
+    # ... and leave the gradients of slots that hold no expert unwritten, as the layer does
+    # (reduce_grad never reads them); with those 58.7 MB per unused slot zeroed beside it
     dwg = ffn.launch_grouped_gemm_wgrad_tn(dg, rows, cu)
-    bw["wgrad_gemm_us_each"] = time_launches(lambda: ffn.launch_grouped_gemm_wgrad_tn(dg, rows, cu, dwg), steps)
+    bw["wgrad_gemm_us_each_zeroing_unused_slots"] = time_launches(
+        lambda: ffn.launch_grouped_gemm_wgrad_tn(dg, rows, cu, dwg), steps)
+    bw["wgrad_gemm_us_each"] = time_launches(
+        lambda: ffn.launch_grouped_gemm_wgrad_tn(dg, rows, cu, dwg, skip_empty_from=G // 2), steps)
     del dg, du, sb, dh, dwg
     gemm_us = bw["dh_gemm_us"] + bw["dual_dgrad_gemm_us"] + 3 * bw["wgrad_gemm_us_each"]
     bw["gemm_TFLOPs"] = 12.0 * used * H * Hp / gemm_us / 1e6

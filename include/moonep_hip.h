@@ -282,12 +282,14 @@ int mep_grouped_gemm_dual_nn(const void* A1, const void* B1, const void* A2, con
  * C[g] [Ma,Nb] fp32 = At[:, rows of g] * Bt[:, rows of g]^T, At [Ma,ld] and
  * Bt [Nb,ld] bf16 with the rank's rows along the contiguous dimension; the rows
  * of group g are [cu_seqlens[g-1], cu_seqlens[g]).  A group without rows gets
- * zeros.  Ma % 128 == 0, Nb % 256 == 0, ld % 128 == 0, ld >= cu_seqlens[G-1].
+ * zeros -- unless its index is >= skip_empty_from, then it is left unwritten
+ * (pass the number of local experts when the slots that hold no expert are
+ * never read; pass G to have every group written).  Ma % 128 == 0, Nb % 256 == 0, ld % 128 == 0, ld >= cu_seqlens[G-1].
  * The fp32 [G,Ma,Nb] result has the layout mep_grad_reduce sums (local experts
  * first, then the slots).  No counterpart in the reference.
  */
 int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int32_t* cu_seqlens, int G,
-                           float* C, int Ma, int Nb, int64_t ld, void* stream);
+                           float* C, int Ma, int Nb, int64_t ld, int skip_empty_from, void* stream);
 
 /*
  * The same weight gradients from the activations as the passes hold them:
@@ -297,7 +299,7 @@ int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int32_t* cu_seq
  * mep_grouped_gemm_wgrad).  No counterpart in the reference.
  */
 int mep_grouped_gemm_wgrad_tn(const void* X1, const void* X2, const int32_t* cu_seqlens, int G,
-                              float* C, int Ma, int Nb, int64_t rows, void* stream);
+                              float* C, int Ma, int Nb, int64_t rows, int skip_empty_from, void* stream);
 
 /*
  * [batch, rows, cols] -> [batch, cols, rows] of bf16 (any 2-byte element);

@@ -57,8 +57,8 @@ _SIGNATURES = {
     "mep_grouped_gemm_dual_nt": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _p]),
     "mep_grouped_gemm_nn": (_i, [_p, _p, _p, _i, _p, _p, _i, _i, _i, _p]),
     "mep_grouped_gemm_dual_nn": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _p]),
-    "mep_grouped_gemm_wgrad": (_i, [_p, _p, _p, _i, _p, _i, _i, _i64, _p]),
-    "mep_grouped_gemm_wgrad_tn": (_i, [_p, _p, _p, _i, _p, _i, _i, _i64, _p]),
+    "mep_grouped_gemm_wgrad": (_i, [_p, _p, _p, _i, _p, _i, _i, _i64, _i, _p]),
+    "mep_grouped_gemm_wgrad_tn": (_i, [_p, _p, _p, _i, _p, _i, _i, _i64, _i, _p]),
     "mep_transpose_bf16": (_i, [_p, _p, _i, _i, _i, _p]),
     "mep_swiglu_bwd": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _p, _p, _i, _i, _p]),
 }

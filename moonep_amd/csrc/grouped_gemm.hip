@@ -69,6 +69,7 @@ struct GemmArgs {
   float* Cf;           // wgrad: [G,M,N] fp32
   int64_t ld;          // row stride of A and B in elements (K, or the row count for wgrad)
   int panel;           // row tiles of a long group that share a sweep over the weight tiles
+  int skip_from;       // wgrad: groups g >= skip_from without rows are left unwritten
 };
 
 enum { kModeScale = 0, kModeSwiglu = 1, kModeDual = 2, kModeWgrad = 3 };
@@ -204,6 +205,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   }
   const size_t K = (size_t)a.ld;
   const bool any = KT > 0;  // a group without rows: its weight gradient is zero
+  if (MODE == kModeWgrad && !any && g >= a.skip_from) return;  // ... and nobody reads it: an unused slot
 
   if (wave >= kConsumers) {
     // =============================== producer ===============================
@@ -687,8 +689,9 @@ __global__ __launch_bounds__(kW2Threads, 1) void wgrad256_kernel(GemmArgs a, Wgr
   };
 
   float* cf = a.Cf + (size_t)g * a.M * a.N;
+  if (KT == 0 && g >= a.skip_from) return;  // an unused slot whose gradient nobody reads
   if (KT == 0) {
-    // a group without rows (an unused slot): its gradient is zero -- whole 1 KB rows of the
+    // a group without rows: its gradient is zero -- whole 1 KB rows of the
     // tile per wave instruction instead of the accumulators' two 128-byte pieces
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
@@ -1066,7 +1069,7 @@ extern "C" int mep_grouped_gemm_dual_nn(const void* A1, const void* B1, const vo
 }
 
 extern "C" int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int32_t* cu_seqlens, int G,
-                                      float* C, int Ma, int Nb, int64_t ld, void* stream) {
+                                      float* C, int Ma, int Nb, int64_t ld, int skip_empty_from, void* stream) {
   MEP_REQUIRE(At && Bt && cu_seqlens && C, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(Ma > 0 && Nb > 0 && G > 0 && ld > 0, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(Ma % kBM == 0 && Nb % kBN == 0 && ld % kBM == 0, MEP_ERR_UNSUPPORTED);
@@ -1077,6 +1080,8 @@ extern "C" int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int3
   a.A = (const uint16_t*)At; a.B = (const uint16_t*)Bt; a.cu = cu_seqlens; a.Cf = C;
   a.M = Ma; a.N = Nb; a.K = 0; a.G = G;
   a.ld = ld;
+  MEP_REQUIRE(skip_empty_from >= 0, MEP_ERR_INVALID_ARG);
+  a.skip_from = skip_empty_from;
   if (Ma % kW2T == 0 && Nb % kW2T == 0 && G % 2 == 0 && (uintptr_t)C % 16 == 0)  // an expert's shapes: 256 x 256 tiles
     return wgrad256_launch<false>(a, (hipStream_t)stream);
   a.mtiles = Ma / kBM;
@@ -1085,7 +1090,8 @@ extern "C" int mep_grouped_gemm_wgrad(const void* At, const void* Bt, const int3
 }
 
 extern "C" int mep_grouped_gemm_wgrad_tn(const void* X1, const void* X2, const int32_t* cu_seqlens, int G,
-                                         float* C, int Ma, int Nb, int64_t rows, void* stream) {
+                                         float* C, int Ma, int Nb, int64_t rows, int skip_empty_from,
+                                         void* stream) {
   MEP_REQUIRE(X1 && X2 && cu_seqlens && C, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(Ma > 0 && Nb > 0 && G > 0 && rows > 0, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(Ma % kW2T == 0 && Nb % kW2T == 0 && G % 2 == 0 && rows % kBM == 0, MEP_ERR_UNSUPPORTED);
@@ -1096,6 +1102,8 @@ extern "C" int mep_grouped_gemm_wgrad_tn(const void* X1, const void* X2, const i
   a.A = (const uint16_t*)X1; a.B = (const uint16_t*)X2; a.cu = cu_seqlens; a.Cf = C;
   a.M = Ma; a.N = Nb; a.K = 0; a.G = G;
   a.ld = rows;
+  MEP_REQUIRE(skip_empty_from >= 0, MEP_ERR_INVALID_ARG);
+  a.skip_from = skip_empty_from;
   return wgrad256_launch<true>(a, (hipStream_t)stream);
 }
 

@@ -181,10 +181,12 @@ def launch_grouped_gemm_dual_nn(a1, w1_kn, a2, w2_kn, cu_seqlens, out=None, *, t
     return out
 
 
-def launch_grouped_gemm_wgrad(at, bt, cu_seqlens, out=None, *, token_padding: int = 128):
+def launch_grouped_gemm_wgrad(at, bt, cu_seqlens, out=None, *, skip_empty_from=None, token_padding: int = 128):
     """Weight gradients from transposed activations: ``out[g] = at[:, rows of g] @
     bt[:, rows of g].T`` -> fp32 [G, Ma, Nb]; at [Ma, M], bt [Nb, M] bf16 with
-    the rank's M rows along the contiguous dimension."""
+    the rank's M rows along the contiguous dimension.  A group without rows gets zeros,
+    unless its index is >= ``skip_empty_from`` (then it is left unwritten: the slots that
+    hold no expert, which ``launch_grad_reduce`` never reads)."""
     _check_groups(at, cu_seqlens, token_padding)
     assert bt.dtype == torch.bfloat16 and bt.is_contiguous() and bt.dim() == 2 and bt.shape[1] == at.shape[1]
     Ma, ld = at.shape
@@ -194,7 +196,8 @@ def launch_grouped_gemm_wgrad(at, bt, cu_seqlens, out=None, *, token_padding: in
         out = torch.empty(G, Ma, Nb, dtype=torch.float32, device=at.device)
     assert out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (G, Ma, Nb)
     rc = _lib.lib().mep_grouped_gemm_wgrad(at.data_ptr(), bt.data_ptr(), cu_seqlens.data_ptr(), G,
-                                           out.data_ptr(), Ma, Nb, ld, _lib.current_stream())
+                                           out.data_ptr(), Ma, Nb, ld, G if skip_empty_from is None else skip_empty_from,
+                                           _lib.current_stream())
     _lib.check(rc, "mep_grouped_gemm_wgrad")
     return out
 
@@ -204,9 +207,10 @@ def wgrad_tn_supported(Ma: int, Nb: int, G: int) -> bool:
     return Ma % 256 == 0 and Nb % 256 == 0 and G % 2 == 0
 
 
-def launch_grouped_gemm_wgrad_tn(x1, x2, cu_seqlens, out=None, *, token_padding: int = 128):
+def launch_grouped_gemm_wgrad_tn(x1, x2, cu_seqlens, out=None, *, skip_empty_from=None, token_padding: int = 128):
     """Weight gradients from the activations as they are: ``out[g] = x1[rows of g].T @
-    x2[rows of g]`` -> fp32 [G, Ma, Nb]; x1 [M, Ma], x2 [M, Nb] bf16, no transposed copies."""
+    x2[rows of g]`` -> fp32 [G, Ma, Nb]; x1 [M, Ma], x2 [M, Nb] bf16, no transposed copies.
+    ``skip_empty_from`` as in ``launch_grouped_gemm_wgrad``."""
     _check_groups(x1, cu_seqlens, token_padding)
     assert x2.dtype == torch.bfloat16 and x2.is_contiguous() and x2.dim() == 2 and x2.shape[0] == x1.shape[0]
     M, Ma = x1.shape
@@ -217,7 +221,8 @@ def launch_grouped_gemm_wgrad_tn(x1, x2, cu_seqlens, out=None, *, token_padding:
         out = torch.empty(G, Ma, Nb, dtype=torch.float32, device=x1.device)
     assert out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (G, Ma, Nb)
     rc = _lib.lib().mep_grouped_gemm_wgrad_tn(x1.data_ptr(), x2.data_ptr(), cu_seqlens.data_ptr(), G,
-                                              out.data_ptr(), Ma, Nb, M, _lib.current_stream())
+                                              out.data_ptr(), Ma, Nb, M, G if skip_empty_from is None else skip_empty_from,
+                                              _lib.current_stream())
     _lib.check(rc, "mep_grouped_gemm_wgrad_tn")
     return out
 
@@ -267,12 +272,15 @@ def grouped_ffn_hip_forward(rows, slots, cu_seqlens, gate_t, up_t, down, *, toke
 
 
 def grouped_ffn_hip_backward(dy, rows, slots, cu_seqlens, gate_t, up_t, down, saved, *,
-                             token_padding: int = 128):
+                             token_padding: int = 128, skip_unused_slots: bool = False):
     """Backward of ``grouped_ffn_hip``: -> (drows [M,H] bf16, dslots [M] fp32 | None,
     dgate_t, dup_t [G,H',H] fp32, ddown [G,H,H'] fp32).  Every GEMM runs on the
     matrix cores through the grouped kernels: the input gradients read the weights
     as they are ([K, N] form), the weight gradients the activations as they are
-    (transposed copies only for shapes the untransposed form does not take)."""
+    (transposed copies only for shapes the untransposed form does not take).
+    ``skip_unused_slots``: the weight gradients of slot groups (the upper half of the
+    groups) that have no rows are left unwritten instead of zeroed -- they belong to slots that
+    hold no expert, which ``launch_grad_reduce`` never reads."""
     gp, up = saved
     dy = dy.contiguous()
     # gradient of the unscaled activation: dy @ down[g], down[g] is [H, H'] = [K, N]
@@ -280,14 +288,16 @@ def grouped_ffn_hip_backward(dy, rows, slots, cu_seqlens, gate_t, up_t, down, sa
     dg, du, hs, dslots = launch_swiglu_bwd(dh, gp, up, slots, cu_seqlens)
     # input gradient: dg @ gate_t[g] + du @ up_t[g], both [H', H] = [K, N]
     drows = launch_grouped_gemm_dual_nn(dg, gate_t, du, up_t, cu_seqlens, token_padding=token_padding)
-    if wgrad_tn_supported(dg.shape[1], rows.shape[1], cu_seqlens.numel()):
+    G = cu_seqlens.numel()
+    kw = dict(token_padding=token_padding, skip_empty_from=G // 2 if skip_unused_slots else None)
+    if wgrad_tn_supported(dg.shape[1], rows.shape[1], G):
         # an expert's shapes: the weight gradients read the activations as they are
-        dgate_t = launch_grouped_gemm_wgrad_tn(dg, rows, cu_seqlens, token_padding=token_padding)
-        dup_t = launch_grouped_gemm_wgrad_tn(du, rows, cu_seqlens, token_padding=token_padding)
-        ddown = launch_grouped_gemm_wgrad_tn(dy, hs, cu_seqlens, token_padding=token_padding)
+        dgate_t = launch_grouped_gemm_wgrad_tn(dg, rows, cu_seqlens, **kw)
+        dup_t = launch_grouped_gemm_wgrad_tn(du, rows, cu_seqlens, **kw)
+        ddown = launch_grouped_gemm_wgrad_tn(dy, hs, cu_seqlens, **kw)
         return drows, dslots, dgate_t, dup_t, ddown
     rows_t, dy_t = transpose_bf16(rows), transpose_bf16(dy)
-    dgate_t = launch_grouped_gemm_wgrad(transpose_bf16(dg), rows_t, cu_seqlens, token_padding=token_padding)
-    dup_t = launch_grouped_gemm_wgrad(transpose_bf16(du), rows_t, cu_seqlens, token_padding=token_padding)
-    ddown = launch_grouped_gemm_wgrad(dy_t, transpose_bf16(hs), cu_seqlens, token_padding=token_padding)
+    dgate_t = launch_grouped_gemm_wgrad(transpose_bf16(dg), rows_t, cu_seqlens, **kw)
+    dup_t = launch_grouped_gemm_wgrad(transpose_bf16(du), rows_t, cu_seqlens, **kw)
+    ddown = launch_grouped_gemm_wgrad(dy_t, transpose_bf16(hs), cu_seqlens, **kw)
     return drows, dslots, dgate_t, dup_t, ddown

@@ -187,7 +187,7 @@ class _GroupExpertFFN(torch.autograd.Function):
             res = ffn.grouped_ffn_hip_backward(
                 g_out[r], ctx.rows_all[r], None if ctx.slots_all is None else ctx.slots_all[r],
                 ctx.cu_all[r], ctx.views[0][r], ctx.views[1][r], ctx.views[2][r], ctx.saved[r],
-                token_padding=tp)
+                token_padding=tp, skip_unused_slots=True)   # grad reduce reads occupied slots only
             drows.append(res[0])
             dslots.append(res[1])
             for acc, g in zip(dw, res[2:]):

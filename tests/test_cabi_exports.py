@@ -110,12 +110,12 @@ def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
     assert lib.mep_grouped_gemm_nn(A, A + 2, A, 4, A, None, 128, 256, 64, None) == -4
     assert lib.mep_grouped_gemm_dual_nn(A, A, None, A, A, 4, A, 128, 256, 64, None) == -1   # second pair missing
     assert lib.mep_grouped_gemm_dual_nn(A, A, A, A, A, 4, A, 128, 128, 64, None) == -2      # N % 256 != 0
-    assert lib.mep_grouped_gemm_wgrad(A, A, A, 4, A, 100, 256, 1024, None) == -2            # Ma % 128 != 0
-    assert lib.mep_grouped_gemm_wgrad(A, A, A, 4, A, 128, 256, 1000, None) == -2            # ld % 128 != 0
-    assert lib.mep_grouped_gemm_wgrad(A, None, A, 4, A, 128, 256, 1024, None) == -1
-    assert lib.mep_grouped_gemm_wgrad_tn(A, A, A, 4, A, 128, 256, 1024, None) == -2         # Ma % 256 != 0
-    assert lib.mep_grouped_gemm_wgrad_tn(A, A, A, 3, A, 256, 256, 1024, None) == -2         # G odd
-    assert lib.mep_grouped_gemm_wgrad_tn(A, A, None, 4, A, 256, 256, 1024, None) == -1
+    assert lib.mep_grouped_gemm_wgrad(A, A, A, 4, A, 100, 256, 1024, 4, None) == -2            # Ma % 128 != 0
+    assert lib.mep_grouped_gemm_wgrad(A, A, A, 4, A, 128, 256, 1000, 4, None) == -2            # ld % 128 != 0
+    assert lib.mep_grouped_gemm_wgrad(A, None, A, 4, A, 128, 256, 1024, 4, None) == -1
+    assert lib.mep_grouped_gemm_wgrad_tn(A, A, A, 4, A, 128, 256, 1024, 4, None) == -2         # Ma % 256 != 0
+    assert lib.mep_grouped_gemm_wgrad_tn(A, A, A, 3, A, 256, 256, 1024, 3, None) == -2         # G odd
+    assert lib.mep_grouped_gemm_wgrad_tn(A, A, None, 4, A, 256, 256, 1024, 4, None) == -1
     assert lib.mep_transpose_bf16(A, A, 1, 64, 64, None) == -1                              # in place
     assert lib.mep_transpose_bf16(A, A + 8192, 1, 64, 96, None) == -2                       # cols % 64 != 0
     assert lib.mep_swiglu_bwd(A, A, A, None, A, 4, A, A, A, None, 128, 100, None) == -2     # N % 8 != 0

@@ -137,6 +137,26 @@ def test_weight_gradients_per_group(cuda, M, Ma, Nb, G, tail):
         tn = ffn.launch_grouped_gemm_wgrad_tn(at.t().contiguous().to(cuda), bt.t().contiguous().to(cuda),
                                               ends.to(cuda))
         assert torch.equal(tn, got)
+    # groups without rows from index G // 2 on are left as they are when the caller says so
+    # (slots that hold no expert); the others do not change
+    half = G // 2
+    kept = torch.full_like(got, 7.0)
+    ffn.launch_grouped_gemm_wgrad(at.to(cuda), bt.to(cuda), ends.to(cuda), kept, skip_empty_from=half)
+    lens = torch.diff(ends, prepend=torch.zeros(1, dtype=torch.int32)).clamp(min=0)
+    for gi in range(G):
+        if gi >= half and int(lens[gi]) == 0:
+            assert bool((kept[gi] == 7.0).all()), f"group {gi} was written"
+        else:
+            assert torch.equal(kept[gi], got[gi]), f"group {gi}"
+    if ffn.wgrad_tn_supported(Ma, Nb, G):
+        kept.fill_(7.0)
+        ffn.launch_grouped_gemm_wgrad_tn(at.t().contiguous().to(cuda), bt.t().contiguous().to(cuda), ends.to(cuda),
+                                         kept, skip_empty_from=half)
+        for gi in range(G):
+            if gi >= half and int(lens[gi]) == 0:
+                assert bool((kept[gi] == 7.0).all()), f"group {gi} was written"
+            else:
+                assert torch.equal(kept[gi], got[gi]), f"group {gi}"
     torch.cuda.synchronize()
     got = got.cpu()
     start, empty = 0, 0
