@@ -2,7 +2,7 @@
 MI355X at S=4096, H=7168, K=8, E=256, R=8, token_padding=128, bf16, routing at
 maxvio ~= 1 (synthetic, seeded).
 
-    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--chain-only]
+    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--sections chain,extras,sweep,weights,ffn]
 
 A step is one pass planner -> dispatch -> combine over one of six rotating
 token sets; the K timed steps are recorded into one HIP graph and replayed
@@ -15,20 +15,25 @@ its COLD, standalone duration (every launch reads a token set that is not in
 any cache); its duration inside the timed steps, where the planner launch has
 already pulled the tokens into the last-level cache, is reported beside it.
 
-The same line carries the other configurations: the chain at maxvio 0 .. 4 on
-both shapes (`maxvio_sweep`), the chain at the configuration of the reference's own
-figure (`reference_figure_config`), prefetch_weight and reduce_grad at
-[32, 7168, 2048] per rank for the planner's own slot table and for a table with
-8 slots per rank (`weights`), the expert-side grouped FFN (`ffn`), each with its
-own `roofline` record, the chain bounded to 32 .. 256 compute units
-(`chain_on_limited_cus`), and the chain with six rotating sets of destination
-shards beside the same chain on one set (`chain_on_rotating_shards`).  The weight
-leg passes three different tensors for the three projections and rotates
-renumbered variants of each table, so no launch re-reads what the one before
-left in the last-level cache.  `--chain-only` skips them.
-
-The CPU baseline is the scalar C restatement of the same chain
-(oracle/mep_oracle.c), timed on the host next to the GPU.
+Sections (all by default; `--sections chain` is the headline alone):
+  chain    config 1 as above and the CPU baseline (the scalar C restatement
+           oracle/mep_oracle.c on the host, same inputs); always measured;
+  extras   the chain bounded to 32 .. 256 compute units (`chain_on_limited_cus`: 32 is
+           the reference's default `num_sms`) and the chain with six rotating sets of
+           destination shards;
+  sweep    the chain at maxvio 0 .. 4 on both shapes with the headline's steps and
+           warm-ups, three timings per point, the fastest kept (`maxvio_sweep`), and
+           the chain at the configuration of the reference's own figure;
+  weights  prefetch_weight (owner push, and the pull of one rank's slots) and
+           reduce_grad at [32, 7168, 2048] per rank on the planner's own slot table
+           and on a table with 8 slots per rank.  Three different tensors for the three
+           projections and renumbered variants of each table in turn, so no launch
+           re-reads what the one before left in the last-level cache;
+  ffn      the expert-side grouped FFN.
+Every section carries its own `roofline` record; the short summary keys
+(`maxvio_sweep_spread_pct`, `maxvio_sweep_chain_us`, the fractions of HBM peak)
+come last in the line.  A 512 MiB device copy runs first: the known-size kernel
+that hardware counters of a profiled run are scaled by.
 """
 
 from __future__ import annotations
@@ -49,17 +54,19 @@ def kernel_source_digest() -> str:
     """Identifies the kernel sources a traffic measurement belongs to."""
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "moonep_amd", "csrc")
-    for name in ("mep_common.h", "dispatch.hip", "combine.hip"):
-        with open(os.path.join(csrc, name), "rb") as f:
-            h.update(f.read())
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h")):
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(f.read())
     return h.hexdigest()[:16]
 
 
-def measured_traffic(kernel: str, grid: int):
-    """(HBM-side bytes per launch, note) for `kernel` from profiles/traffic.json: L2
-    fetches + writes counted by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by the
-    factors a 512 MiB copy gives.  The figure is only used when the file was made from the
-    kernel sources and the launch grid that run now; otherwise (None, why)."""
+def measured_traffic(key: str, grid=None):
+    """(HBM-side bytes per launch, note) for the record `key` of profiles/traffic.json: L2
+    fetches + writes counted by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this program and
+    scaled by the factors its 512 MiB copy gives.  The figure is only used when the file was
+    made from the kernel sources (and, where given, the launch grid) that run now; otherwise
+    (None, why)."""
     try:
         with open(TRAFFIC_FILE) as f:
             rec = json.load(f)
@@ -67,12 +74,15 @@ def measured_traffic(kernel: str, grid: int):
         return None, f"no traffic record: {exc}"
     if rec.get("source_digest") != kernel_source_digest():
         return None, "profiles/traffic.json was measured on other kernel sources: re-run the PMC profile"
-    k = rec.get("kernels", {}).get(kernel)
+    k = rec.get("kernels", {}).get(key)
     if k is None:
-        return None, f"profiles/traffic.json has no entry for {kernel}"
-    if int(k.get("grid", -1)) != int(grid):
-        return None, f"profiles/traffic.json: {kernel} was measured with grid {k.get('grid')}, not {grid}"
+        return None, f"profiles/traffic.json has no entry for {key}"
+    if grid is not None and int(k.get("grid", -1)) != int(grid):
+        return None, f"profiles/traffic.json: {key} was measured with grid {k.get('grid')}, not {grid}"
     return float(k["fetch_bytes"]) + float(k["write_bytes"]), None
+
+
+SECTIONS = ("chain", "extras", "sweep", "weights", "ffn")
 
 
 def parse():
@@ -80,27 +90,19 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--chain-only", action="store_true",
-                    help="config 1 only: skip the maxvio sweep, prefetch / grad reduce and the FFN")
-    ap.add_argument("--full", action="store_true", help="accepted for older command lines; everything runs by default")
-    ap.add_argument("--write-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
-                    help="no GPU work: turn the counter_collection.csv files of two rocprofv3 --pmc runs of "
-                         "`bench.py --profile-kernels` (FETCH_SIZE, WRITE_SIZE) into profiles/traffic.json")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--ffn-only", action="store_true",
-                    help="only the expert FFN section (grouped GEMMs, forward and backward), for profiling it")
-    ap.add_argument("--no-limited-cus", action="store_true",
-                    help="skip the leg that times the chain on CU-masked streams (under rocprofv3 a process "
-                         "that still holds such a stream has crashed in the profiler's exit handlers)")
-    ap.add_argument("--profile-kernels", action="store_true",
-                    help="for rocprofv3: a few plain launches of each kernel and of a 512 MiB "
-                         "torch copy (the known-size kernel counters are scaled by); no JSON")
-    ap.add_argument("--profile-weights", action="store_true",
-                    help="for rocprofv3 --pmc: three rounds of a 512 MiB copy, prefetch_weight and reduce_grad "
-                         "on the table with 8 slots per rank, then exit")
+    ap.add_argument("--sections", default=",".join(SECTIONS),
+                    help="comma-separated subset of chain,extras,sweep,weights,ffn (default: all); the headline "
+                         "chain is always measured")
+    ap.add_argument("--chain-only", action="store_true", help="same as --sections chain")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--maxvio", type=float, default=1.0)
     ap.add_argument("--seed", type=int, default=2024)
-    return ap.parse_args()
+    args = ap.parse_args()
+    args.sections = {"chain"} if args.chain_only else set(x for x in args.sections.split(",") if x)
+    unknown = args.sections - set(SECTIONS)
+    if unknown:
+        ap.error(f"unknown section(s): {sorted(unknown)}")
+    return args
 
 
 def hbm_roofline(kernel, algorithmic_bytes, us, traffic=None, **extra):
@@ -373,45 +375,6 @@ def chain_on_rotating_shards(ch, steps, nsets=6):
     return out
 
 
-def profile_weights():
-    """Launches for a counter run: a 512 MiB copy (the scale of FETCH_SIZE / WRITE_SIZE), then
-    prefetch_weight (3 projections) and reduce_grad (one projection) at [32, 7168, 2048], R = 8,
-    every rank hosting 8 remote experts, three times on three renumbered tables."""
-    import numpy as np
-    import torch
-
-    from moonep_amd.grad_reduce import launch_grad_reduce
-    from moonep_amd.prefetch import launch_prefetch
-
-    E, R, H, Hp = 256, 8, 7168, 2048
-    epn, rank = E // R, 7
-    dev = torch.device("cuda", 0)
-    ring = -np.ones((R, epn), dtype=np.int64)
-    for d in range(R):
-        for b in range(8):
-            ring[d, b] = ((d + 1 + b) % R) * epn + (d * 8 + b) % epn
-    local = [(torch.randn(epn, H, Hp, device=dev) * 0.02).to(torch.bfloat16) for _ in range(3)]
-    pool = [torch.empty(R, epn, H, Hp, dtype=torch.bfloat16, device=dev) for _ in range(3)]
-    grad = torch.zeros(epn, H, Hp, dtype=torch.float32, device=dev)
-    red = torch.randn(R, epn, H, Hp, dtype=torch.float32, device=dev) * 1e-3
-    src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).view(torch.float32)
-    dst = torch.empty_like(src)
-    for v in range(3):
-        e = ring.copy()
-        m = e >= 0
-        e[m] = (e[m] // epn) * epn + (e[m] % epn + 11 * v) % epn
-        etc = torch.from_numpy(np.roll(e, 5 * v, axis=1).astype("int32")).to(dev)
-        dst.copy_(src)
-        launch_prefetch(tuple(local), tuple(pool), etc, rank=rank)
-        launch_grad_reduce(grad, red, etc, rank=rank)
-        torch.cuda.synchronize()
-    per = H * Hp
-    print(json.dumps({"profile_weights": {"launches_each": 3, "prefetch_bytes": 3 * 16 * per * 2,
-                                          "prefetch_read_bytes": 3 * 8 * per * 2,
-                                          "grad_reduce_bytes": 32 * per * 4,
-                                          "grad_reduce_read_bytes": 16 * per * 4}}), file=sys.stderr)
-
-
 def cpu_baseline(ch, budget_s=10.0):
     """Scalar C port of plan + dispatch + combine on the same inputs, host cores."""
     import numpy as np
@@ -505,15 +468,16 @@ def gpu_plan_all_ranks(S, K, E, R, tp, topk, tpe):
 
 
 def bench_weights(seed, steps, cpu=True):
-    """prefetch_weight (3 projections, one launch) and reduce_grad (one projection) at
-    H=7168, H'=2048, epn=32, R=8 for two slot tables: the planner's own at maxvio~1
-    (busiest owner) and a denser ring (every rank hosts 8 remote experts)."""
+    """prefetch_weight (3 projections, one launch: the owner's push, and the pull of one
+    rank's slots from all owners) and reduce_grad (one projection) at H=7168, H'=2048,
+    epn=32, R=8 for two slot tables: the planner's own at maxvio~1 (busiest owner /
+    fullest rank) and a denser ring (every rank hosts 8 remote experts)."""
     import numpy as np
     import torch
 
     from moonep_amd import routing
     from moonep_amd.grad_reduce import launch_grad_reduce
-    from moonep_amd.prefetch import launch_prefetch
+    from moonep_amd.prefetch import launch_prefetch, launch_prefetch_pull
 
     S, K, E, R, H, Hp = 4096, 8, 256, 8, 7168, 2048
     epn = E // R
@@ -531,6 +495,8 @@ def bench_weights(seed, steps, cpu=True):
     # 256 MB last-level cache from the projection or the launch before it
     local = [(torch.randn(epn, H, Hp, device=dev) * 0.02).to(torch.bfloat16) for _ in range(3)]
     pool = [torch.empty(R, epn, H, Hp, dtype=torch.bfloat16, device=dev) for _ in range(3)]
+    # every rank's local experts side by side, for the pull (contents do not matter to a copy)
+    owners = [torch.empty(R, epn, H, Hp, dtype=torch.bfloat16, device=dev) for _ in range(3)]
     res = {"plan_maxvio": mv}
     tables = {"planner": planned, "ring8": ring}
     NROT = 3
@@ -561,8 +527,22 @@ def bench_weights(seed, steps, cpu=True):
         res[name] = {"rank": rank, "slots": n_slots, "active_experts": active,
                      "own_occupied_slots": own_slots, "prefetch_us_3proj": us,
                      "prefetch_bytes": by, "prefetch_GBps": by / us / 1e3 if by else 0.0,
-                     "prefetch_roofline": hbm_roofline("prefetch_kernel", by, us)}
-    del local, pool
+                     "prefetch_roofline": hbm_roofline("prefetch_kernel", by, us,
+                                                       measured_traffic(f"prefetch_kernel@{name}")[0])}
+        # the pull view: the fullest rank's slots from all owners in one launch
+        pull_slots, pull_rank = max((int((etc_np[r] >= 0).sum()), r) for r in range(R))
+
+        def pl():
+            k[0] += 1
+            launch_prefetch_pull(tuple(owners), tuple(pool), variants[k[0] % NROT], rank=pull_rank)
+
+        us = time_launches(pl, steps)
+        by = 3 * 2 * pull_slots * per * 2       # every occupied slot: one expert read, one written
+        res[name].update({"pull_rank": pull_rank, "pull_slots": pull_slots, "prefetch_pull_us_3proj": us,
+                          "prefetch_pull_bytes": by, "prefetch_pull_GBps": by / us / 1e3 if by else 0.0,
+                          "prefetch_pull_roofline": hbm_roofline(
+                              "prefetch_pull_kernel", by, us, measured_traffic(f"prefetch_pull_kernel@{name}")[0])})
+    del local, pool, owners
     torch.cuda.empty_cache()
     grad = torch.zeros(epn, H, Hp, dtype=torch.float32, device=dev)
     red = torch.randn(R, epn, H, Hp, dtype=torch.float32, device=dev) * 1e-3
@@ -577,7 +557,8 @@ def bench_weights(seed, steps, cpu=True):
         by = (n_slots + 2 * active + own_slots) * per * 4   # slots read, grads read+written, clears
         res[name].update({"grad_reduce_us": us, "grad_reduce_bytes": by,
                           "grad_reduce_GBps": by / us / 1e3 if by else 0.0,
-                          "grad_reduce_roofline": hbm_roofline("grad_reduce_kernel", by, us)})
+                          "grad_reduce_roofline": hbm_roofline(
+                              "grad_reduce_kernel", by, us, measured_traffic(f"grad_reduce_kernel@{name}")[0])})
     del grad, red
     torch.cuda.empty_cache()
     if not cpu:
@@ -675,58 +656,12 @@ def bench_ffn(seed, steps):
         "rows_in_groups": used, "NvS": NvS, "groups": G, "maxvio": mv, "backward": bw,
         "swiglu_gate_up_us": t1, "swiglu_gate_up_TFLOPs": f1 / t1 / 1e6,
         "down_us": t2, "down_TFLOPs": f2 / t2 / 1e6,
-        "roofline": {"bound": "mfma", "kernel": "grouped_gemm_nt_kernel", "achieved": (f1 + f2) / (t1 + t2) / 1e6,
-                     "peak": peak, "unit": "TFLOP/s", "frac": (f1 + f2) / (t1 + t2) / 1e6 / peak, "traffic": None},
+        "roofline": {"bound": "mfma", "kernel": "grouped_gemm256_kernel (SwiGLU gate/up + down)",
+                     "achieved": (f1 + f2) / (t1 + t2) / 1e6, "peak": peak, "unit": "TFLOP/s",
+                     "frac": (f1 + f2) / (t1 + t2) / 1e6 / peak,
+                     "traffic": measured_traffic("grouped_gemm_forward")[0]},
         "library_dense_gemm_TFLOPs": 2.0 * used * H * Hp / t3 / 1e6,
     }
-
-
-def write_traffic(fetch_csv, write_csv):
-    """profiles/traffic.json from the counter CSVs of two rocprofv3 --pmc runs of
-    `bench.py --profile-kernels` (one with FETCH_SIZE, one with WRITE_SIZE)."""
-    import csv
-
-    def per_kernel(path, counter):
-        acc = {}
-        with open(path) as f:
-            for row in csv.DictReader(f):
-                if row["Counter_Name"] != counter:
-                    continue
-                # launches of one kernel with another grid (the runtime's small staging copies
-                # share the name of the 512 MiB copy) are records of their own
-                key = (row["Kernel_Name"], int(row["Grid_Size"]))
-                v = acc.setdefault(key, {"sum": 0.0, "n": 0, "grid": int(row["Grid_Size"]),
-                                         "wg": int(row["Workgroup_Size"])})
-                v["sum"] += float(row["Counter_Value"])
-                v["n"] += 1
-        return {k: (v["sum"] / v["n"], v["grid"] // v["wg"], v["n"]) for k, v in acc.items()}
-
-    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
-    copy = [k for k in fetch if "copyBuffer" in k[0]]
-    assert copy, "the run must contain the 512 MiB copy the counters are scaled by"
-    known_kib = 512 * 1024
-    f_scale = known_kib / max(v[0] for k, v in fetch.items() if k in copy)
-    w_scale = known_kib / max(v[0] for k, v in write.items() if k in copy)
-    kernels = {}
-    for short in ("dispatch_kernel", "combine_kernel", "plan_kernel"):
-        names = [k for k in fetch if short in k[0]]
-        if not names:
-            continue
-        k = names[0]
-        kernels[short] = {"name": k[0], "grid": fetch[k][1], "launches": fetch[k][2],
-                          "fetch_bytes": fetch[k][0] * 1024 * f_scale,
-                          "write_bytes": write[k][0] * 1024 * w_scale}
-    rec = {"source_digest": kernel_source_digest(),
-           "made_by": "python bench.py --write-traffic <fetch csv> <write csv> after two runs of "
-                      "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -- python3 bench.py --profile-kernels",
-           "scale": {"FETCH_SIZE": f_scale, "WRITE_SIZE": w_scale,
-                     "from": "a 512 MiB device-to-device copy in the same run"},
-           "workload": "config 1: S=4096 H=7168 K=8 E=256 R=8 token_padding=128 maxvio~1, rank 0",
-           "kernels": kernels}
-    with open(TRAFFIC_FILE, "w") as f:
-        json.dump(rec, f, indent=1)
-        f.write("\n")
-    print(json.dumps(rec))
 
 
 def dispatch_grid(S, K, E, R, tp):
@@ -736,11 +671,66 @@ def dispatch_grid(S, K, E, R, tp):
     return (S * K + 3) // 4 + (2 * (E // R) * zpg if tp > 1 else 0)
 
 
+def sweep_point(ch, steps, warmup, repeats=3):
+    """One point of the maxvio sweep, timed like the headline: `warmup` steps, then the
+    `steps` steps of one HIP graph between two events, `repeats` times; returns (the
+    per-step microseconds of every repeat, the kernels' durations inside an eager chain)."""
+    import torch
+
+    for i in range(warmup):
+        ch.step(i)
+    torch.cuda.synchronize()
+    big = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(big):
+        for i in range(steps):
+            j = i % len(ch.hidden)
+            ch.plan_fn(j); ch.dispatch_fn(j); ch.combine_fn(j)
+    big.replay()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    times = []
+    for _ in range(repeats):
+        a.record()
+        big.replay()
+        b.record()
+        b.synchronize()
+        times.append(a.elapsed_time(b) * 1e3 / steps)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+    for i in range(steps):
+        j = i % len(ch.hidden)
+        evs[i][0].record(); ch.plan_fn(j)
+        evs[i][1].record(); ch.dispatch_fn(j)
+        evs[i][2].record(); ch.combine_fn(j)
+        evs[i][3].record()
+    torch.cuda.synchronize()
+    skip = min(2, steps - 1)
+    in_chain = [sum(e[q].elapsed_time(e[q + 1]) for e in evs[skip:]) * 1e3 / (steps - skip) for q in range(3)]
+    return times, in_chain
+
+
+def calibration_copy(repeats=3):
+    """A 512 MiB device-to-device copy: the kernel of known size (reads 512 MiB, writes
+    512 MiB) that FETCH_SIZE / WRITE_SIZE of a counter run of this program are scaled by."""
+    import torch
+
+    src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda").view(torch.float32)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(repeats):
+        dst.copy_(src)
+    b.record()
+    b.synchronize()
+    us = a.elapsed_time(b) * 1e3 / repeats
+    del src, dst
+    torch.cuda.empty_cache()
+    return {"bytes_each_way": 512 << 20, "us": us, "GBps": 2 * (512 << 20) / us / 1e3}
+
+
 def main():
     args = parse()
-    if args.write_traffic:
-        write_traffic(*args.write_traffic)
-        return
     if args.gpus != 1:
         print("bench.py measures one rank's share on ONE GPU; --gpus > 1 is not part of this "
               "build (no collectives, no sharding).", file=sys.stderr)
@@ -748,24 +738,9 @@ def main():
     import torch
 
     torch.cuda.set_device(0)
-    if args.profile_weights:
-        profile_weights()
-        return
-    if args.ffn_only:
-        print(json.dumps({"ffn": bench_ffn(args.seed, max(2, args.steps // 4))}))
-        return
+    copy_rec = calibration_copy()
     S, H, K, E, R, tp, rank = 4096, 7168, 8, 256, 8, 128, 0
     ch = Chain(S, H, K, E, R, tp, rank, args.maxvio, args.seed)
-    if args.profile_kernels:
-        src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda").view(torch.float32)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)            # reads 512 MiB, writes 512 MiB
-            ch.plan_fn(); ch.dispatch_fn(0); ch.combine_fn(0)
-            torch.cuda.synchronize()
-        print("profile-kernels: 3 x (copy 512MiB, plan, dispatch, combine) launched", file=sys.stderr)
-        ch.destroy()
-        return
     wall_ms, ev_ms, per = measure_chain(ch, args.steps, args.warmup)
     by = ch.bytes_one_way()
     value = 2 * by / (wall_ms * 1e-3) / 1e9
@@ -785,8 +760,13 @@ def main():
         "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "config 1: single-rank dispatch+combine, S=4096 H=7168 K=8 E=256 R=8 "
-                               "token_padding=128, the timed plan->dispatch->combine steps recorded in one HIP graph",
+                               "token_padding=128, the timed plan->dispatch->combine steps recorded in one HIP graph; "
+                               "kernels on the whole GPU (the reference's default bounds them to 32 SMs: see "
+                               "chain_on_limited_cus)",
                    "maxvio": round(ch.maxvio, 3), "seed": args.seed, "rank": rank},
+        "roofline": roof,
+        "combine_roofline": hbm_roofline("combine_kernel", by, per["combine_us"],
+                                         measured_traffic("combine_kernel", S * 7 // 4)[0]),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "graph_ms_per_step_events": ev_ms,
         "ms_per_step_one_graph_replay_per_step": per["single_replay_ms"],
@@ -797,61 +777,77 @@ def main():
         "combine_weighted_us": per["combine_weighted_us"],
         "dispatch_GBps": per["dispatch_GBps"], "combine_GBps": per["combine_GBps"],
         "dispatch_us_warm_input": per["dispatch_us_warm_input"],
-        "dispatch_pct_hbm_peak": 100.0 * per["dispatch_GBps"] / HBM_PEAK_GBPS,
-        "combine_pct_hbm_peak": 100.0 * per["combine_GBps"] / HBM_PEAK_GBPS,
-        "roofline": roof,
-        "combine_roofline": hbm_roofline("combine_kernel", by, per["combine_us"],
-                                         measured_traffic("combine_kernel", S * 7 // 4)[0]),
+        "calibration_copy": copy_rec,
     }
-    if not (args.chain_only or args.no_limited_cus):
-        line["chain_on_limited_cus"] = chain_on_limited_cus(ch, max(5, args.steps // 2))
-    if not args.chain_only:
-        line["chain_on_rotating_shards"] = chain_on_rotating_shards(ch, args.steps)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(ch)
+    sub_steps = max(5, args.steps // 2)
+    if "extras" in args.sections:
+        line["chain_on_limited_cus"] = chain_on_limited_cus(ch, sub_steps)
+        line["chain_on_rotating_shards"] = chain_on_rotating_shards(ch, args.steps)
     ch.destroy()
     torch.cuda.empty_cache()
-    if not args.chain_only:
-        sweep = {}
-        sub_steps = max(5, args.steps // 2)
+    tail = {}          # short summary keys, appended last
+    if "sweep" in args.sections:
+        sweep, spread, chain_us = {}, {}, {}
         for shape in ((4096, 7168, 256), (8192, 4096, 128)):
-            chain_us = []
+            tag = f"S{shape[0]}_H{shape[1]}_E{shape[2]}"
+            best = []
             for mv in (0.0, 0.5, 1.0, 2.0, 4.0):
                 c2 = Chain(shape[0], shape[1], K, shape[2], R, tp, rank, mv, args.seed)
-                w2, e2, p2 = measure_chain(c2, sub_steps, 2, kernels=False)
+                times, p2 = sweep_point(c2, args.steps, args.warmup)
+                us = min(times)
                 b2 = c2.bytes_one_way()
-                sweep[f"S{shape[0]}_H{shape[1]}_E{shape[2]}_maxvio{mv}"] = {
-                    "maxvio": round(c2.maxvio, 3), "chain_us": w2 * 1e3,
-                    "GBps": 2 * b2 / w2 / 1e6, "pct_hbm_peak": 2 * b2 / w2 / 1e6 / HBM_PEAK_GBPS * 100.0,
-                    "plan_us_in_chain": p2["plan_us_in_chain"],
-                    "dispatch_us_in_chain": p2["dispatch_us_in_chain"],
-                    "combine_us_in_chain": p2["combine_us_in_chain"]}
-                chain_us.append(w2 * 1e3)
+                sweep[f"{tag}_maxvio{mv}"] = {
+                    "maxvio": round(c2.maxvio, 3), "chain_us": us, "chain_us_repeats": times,
+                    "GBps": 2 * b2 / us / 1e3, "pct_hbm_peak": 2 * b2 / us / 1e3 / HBM_PEAK_GBPS * 100.0,
+                    "plan_us_in_chain": p2[0], "dispatch_us_in_chain": p2[1], "combine_us_in_chain": p2[2]}
+                best.append(round(us, 1))
                 c2.destroy()
                 torch.cuda.empty_cache()
-            sweep[f"S{shape[0]}_H{shape[1]}_E{shape[2]}_spread_pct"] = \
-                100.0 * (max(chain_us) - min(chain_us)) / min(chain_us)
+            chain_us[tag] = best
+            spread[tag] = round(100.0 * (max(best) - min(best)) / min(best), 2)
+        sweep["timing"] = (f"{args.steps} steps in one HIP graph after {args.warmup} warm-up steps, 3 replays per "
+                           "point, the fastest kept; maxvio 0, 0.5, 1, 2, 4 in that order")
         line["maxvio_sweep"] = sweep
+        tail["maxvio_sweep_chain_us"] = chain_us
+        tail["maxvio_sweep_spread_pct"] = spread
         # the configuration of the reference's own figure (figure/comm_vs_deepep.png: ep = 8,
         # E = 384, H = 7168, K = 8, S = 8192; H20, read off the chart: planning ~40-50 us,
         # dispatch + epilogue ~1835-1855 us, combine ~1932-1975 us, both bound by NVLink)
         c3 = Chain(8192, 7168, K, 384, R, tp, rank, 1.0, args.seed, nsets=3)
-        w3, e3, p3 = measure_chain(c3, sub_steps, 2, kernels=False)
+        t3, p3 = sweep_point(c3, sub_steps, 2)
+        w3 = min(t3)
         b3 = c3.bytes_one_way()
         line["reference_figure_config"] = {
             "workload": "S=8192 H=7168 K=8 E=384 R=8 token_padding=128, one rank's share on one GPU (HBM-bound; "
                         "the reference's figure is NVLink-bound on H20: not the same quantity)",
-            "maxvio": round(c3.maxvio, 3), "chain_us": w3 * 1e3, "GBps": 2 * b3 / w3 / 1e6,
-            "pct_hbm_peak": 2 * b3 / w3 / 1e6 / HBM_PEAK_GBPS * 100.0,
-            "plan_us_in_chain": p3["plan_us_in_chain"], "dispatch_us_in_chain": p3["dispatch_us_in_chain"],
-            "combine_us_in_chain": p3["combine_us_in_chain"],
+            "maxvio": round(c3.maxvio, 3), "chain_us": w3, "GBps": 2 * b3 / w3 / 1e3,
+            "pct_hbm_peak": 2 * b3 / w3 / 1e3 / HBM_PEAK_GBPS * 100.0,
+            "plan_us_in_chain": p3[0], "dispatch_us_in_chain": p3[1], "combine_us_in_chain": p3[2],
             "reference_read_off_its_figure_us": {"planning": "40-50", "dispatch_and_epilogue": "1835-1855",
                                                  "combine": "1932-1975", "hardware": "H20, 8 GPUs, NVLink"}}
         c3.destroy()
         torch.cuda.empty_cache()
-        line["weights"] = bench_weights(args.seed, max(5, args.steps // 2), cpu=not args.no_cpu)
+    if "weights" in args.sections:
+        line["weights"] = bench_weights(args.seed, sub_steps, cpu=not args.no_cpu)
         torch.cuda.empty_cache()
-        line["ffn"] = bench_ffn(args.seed, max(5, args.steps // 2))
+        tail["weights_frac_of_hbm_peak"] = {
+            f"{op}@{name}": round(line["weights"][name][f"{op}_roofline"]["frac"], 3)
+            for name in ("planner", "ring8") for op in ("prefetch", "prefetch_pull", "grad_reduce")}
+    if "ffn" in args.sections:
+        line["ffn"] = bench_ffn(args.seed, sub_steps)
+        tail["ffn_frac_of_mfma_peak"] = round(line["ffn"]["roofline"]["frac"], 3)
+    # the summary comes last, so that the end of the line shows it
+    tail.update({
+        "chain_us": round(wall_ms * 1e3, 1), "plan_us_summary": round(per["plan_us"], 1),
+        "dispatch_us_cold": round(per["dispatch_us"], 1), "dispatch_us_in_chain_summary": round(per["dispatch_us_in_chain"], 1),
+        "combine_us_summary": round(per["combine_us"], 1),
+        "dispatch_pct_hbm_peak": round(100.0 * per["dispatch_GBps"] / HBM_PEAK_GBPS, 1),
+        "combine_pct_hbm_peak": round(100.0 * per["combine_GBps"] / HBM_PEAK_GBPS, 1),
+        "chain_pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 1),
+        "roofline_frac": round(roof["frac"], 3)})
+    line.update(tail)
     print(json.dumps(line))
 
 

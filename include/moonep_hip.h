@@ -54,8 +54,23 @@ extern "C" {
                                    weighted top-k sum that callers otherwise apply on the
                                    expert side                                              */
 
+/* major*10000 + minor*100 + patch.  200: mep_grad_reduce takes `flags` before `stream`,
+ * mep_dispatch_epilogue / mep_combine_prologue take `max_cus` before `stream`; mep_init,
+ * mep_prefetch_pull and mep_set_gemm_row_tile exist.  A binding written against another
+ * version must refuse to load the library. */
 int mep_version(void);
 const char* mep_strerror(int code);
+
+/*
+ * Per-device set-up that must not happen under stream capture: opts every kernel that
+ * uses more than 64 KB of dynamic LDS in (hipFuncSetAttribute).  Call it once per device,
+ * with that device current, before the first launch that may be captured into a graph
+ * (the Python binding calls it when it loads the library and when a Buffer is made).
+ * Idempotent and thread-safe; launches on a device nobody initialised do it themselves,
+ * which only works outside capture.  No counterpart in the reference (its kernels are
+ * JIT-compiled per shape on first use, moonep/dispatch.py:704-720).
+ */
+int mep_init(void);
 
 /*
  * A stream whose kernels run on at most `num_cus` compute units (a CU mask on
@@ -169,14 +184,18 @@ int mep_build_dedup_static(const int32_t* dst_RN, int rank, int S, int K, int R,
                            void* stream);
 
 /* primary row -> its duplicate rows, in place on one rank's shard.
- * Replaces launch_dispatch_epilogue (reference moonep/dispatch_epilogue.py:366-415). */
+ * Replaces launch_dispatch_epilogue (reference moonep/dispatch_epilogue.py:366-415).
+ * max_cus > 0 bounds the launch to that many workgroups, hence compute units -- the
+ * grid the reference sizes from MOONEP_NUM_SMS_DEDUP (moonep/api.py:100-120,
+ * dispatch_epilogue.py:366-415); max_cus <= 0: the whole GPU.  Results do not depend on it. */
 int mep_dispatch_epilogue(void* shard_NvS_H, const int32_t* dup_groups, const int32_t* dup_loffs,
-                          const int32_t* dup_counts, int NvS, int H, void* stream);
+                          const int32_t* dup_counts, int NvS, int H, int max_cus, void* stream);
 
 /* fp32 sum of primary + duplicates -> bf16 -> primary row, in place.
- * Replaces launch_combine_prologue (reference moonep/combine_prologue.py:544-599). */
+ * Replaces launch_combine_prologue (reference moonep/combine_prologue.py:544-599).
+ * max_cus as for mep_dispatch_epilogue. */
 int mep_combine_prologue(void* shard_NvS_H, const int32_t* dup_groups, const int32_t* dup_loffs,
-                         const int32_t* dup_counts, int NvS, int H, void* stream);
+                         const int32_t* dup_counts, int NvS, int H, int max_cus, void* stream);
 
 /*
  * Top-k unpermute + K-sum + weight gather.  Replaces launch_combine
@@ -201,6 +220,22 @@ int mep_combine(const void* shards, int64_t shard_stride_rows, const float* wslo
 int mep_prefetch(int ntensors, const void* const* local, void* const* pool,
                  const int64_t* rank_stride_bytes, const int64_t* bytes_per_expert,
                  const int32_t* experts_to_copy, int rank, int epn, int R, void* stream);
+
+/*
+ * Pull view of the same prefetch: fills the occupied slots of ONE rank from all owners in
+ * one launch, pool_t[rank][b] = owners_t[e / epn][e % epn] for every b with
+ * e = experts_to_copy[rank, b] >= 0 -- what R owner pushes leave in rank's slots, and the
+ * compact [2*epn, ...] compute view of a rank when one GPU holds every owner's experts.
+ * The reference has no such launcher (its ranks push, moonep/prefetch.py:428-447); its
+ * per-rank check of the result is tests/test_prefetch.py:448-464.
+ *   owners[t]: expert le of owner o at owners[t] + o*owner_stride_bytes[t] +
+ *   le*bytes_per_expert[t]; pool as in mep_prefetch; all four arrays are HOST arrays of
+ *   length ntensors (3 or 6).  Slots with -1 and other ranks' slots are not touched.
+ */
+int mep_prefetch_pull(int ntensors, const void* const* owners, const int64_t* owner_stride_bytes,
+                      void* const* pool, const int64_t* rank_stride_bytes,
+                      const int64_t* bytes_per_expert, const int32_t* experts_to_copy, int rank,
+                      int epn, int R, void* stream);
 
 /*
  * fp32 slot reduction.  Replaces launch_grad_reduce (reference
@@ -236,6 +271,10 @@ int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t rank_stride_e
 int mep_grouped_gemm_nt(const void* A, const void* B, const void* B_up, const int32_t* cu_seqlens,
                         int G, void* C, const float* row_scale, int M, int N, int K, int swiglu,
                         void* stream);
+
+/* Test hook: force the row tiling of the grouped GEMMs (128 or 256 rows; 0 = choose by
+ * shape, the default).  Process-wide.  No counterpart in the reference. */
+int mep_set_gemm_row_tile(int rows);
 
 /*
  * The same fused gate/up GEMM, storing the two pre-activations beside the

@@ -33,6 +33,7 @@ _sz = C.c_size_t
 
 _SIGNATURES = {
     "mep_version": (_i, []),
+    "mep_init": (_i, []),
     "mep_strerror": (C.c_char_p, [_i]),
     "mep_stream_create_limited": (_i, [_i, C.POINTER(_p)]),
     "mep_stream_destroy": (_i, [_p]),
@@ -46,12 +47,15 @@ _SIGNATURES = {
     "mep_dedup_scratch_bytes": (_sz, [_i, _i]),
     "mep_build_dedup": (_i, [_p, _i, _i, _i, _i, _i, _p, _p, _p, _p, _sz, _p]),
     "mep_build_dedup_static": (_i, [_p, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
-    "mep_dispatch_epilogue": (_i, [_p, _p, _p, _p, _i, _i, _p]),
-    "mep_combine_prologue": (_i, [_p, _p, _p, _p, _i, _i, _p]),
+    "mep_dispatch_epilogue": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
+    "mep_combine_prologue": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
     "mep_combine": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "mep_prefetch": (_i, [_i, C.POINTER(_p), C.POINTER(_p), C.POINTER(_i64), C.POINTER(_i64),
                           _p, _i, _i, _i, _p]),
+    "mep_prefetch_pull": (_i, [_i, C.POINTER(_p), C.POINTER(_i64), C.POINTER(_p), C.POINTER(_i64),
+                               C.POINTER(_i64), _p, _i, _i, _i, _p]),
     "mep_grad_reduce": (_i, [_p, _p, _i64, _p, _i, _i, _i, _i64, C.c_uint, _p]),
+    "mep_set_gemm_row_tile": (_i, [_i]),
     "mep_grouped_gemm_nt": (_i, [_p, _p, _p, _p, _i, _p, _p, _i, _i, _i, _i, _p]),
     "mep_grouped_swiglu_nt": (_i, [_p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _p]),
     "mep_grouped_gemm_dual_nt": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _p]),
@@ -64,6 +68,10 @@ _SIGNATURES = {
 }
 
 EXPORTS = tuple(_SIGNATURES)
+ABI_VERSION = 200     # mep_version() of the library these signatures were written against
+# hipError_t values that say "no usable GPU in this process" (hipErrorNoDevice,
+# hipErrorInvalidDevice, hipErrorInsufficientDriver): loading the library there is fine
+_NO_GPU_CODES = (100, 101, 35)
 
 
 def lib():
@@ -82,8 +90,22 @@ def lib():
                     fn = getattr(handle, name)
                     fn.restype = res
                     fn.argtypes = args
+                found = handle.mep_version()
+                if found != ABI_VERSION:
+                    raise RuntimeError(
+                        f"{LIB_PATH} has ABI version {found}, this binding needs {ABI_VERSION}: "
+                        "rebuild it with `python -m moonep_amd.build`")
+                # LDS opt-ins of the current device, outside any stream capture
+                rc = handle.mep_init()
+                if rc != 0 and rc not in _NO_GPU_CODES:
+                    raise RuntimeError(f"mep_init failed: {handle.mep_strerror(rc).decode()} (code {rc})")
                 _lib = handle
     return _lib
+
+
+def init_device() -> None:
+    """``mep_init`` for the current device (a process may use several)."""
+    check(lib().mep_init(), "mep_init")
 
 
 def check(code: int, what: str) -> None:

@@ -73,26 +73,55 @@ from .prefetch import _ELEM_TYPES, launch_prefetch
 logger = logging.getLogger(__name__)
 
 
+def _lib_init_device() -> None:
+    from . import _lib
+    _lib.init_device()
+
+
 def _align_up(x: int, alignment: int) -> int:
     return ((x + alignment - 1) // alignment) * alignment
 
 
-def _validate_rank_strided_pool(pool: torch.Tensor) -> int:
-    """Stride (in elements) between the ranks of a pool.  Each rank's payload is
-    one contiguous block; blocks may be padded apart but not overlap, start on
-    16-byte boundaries and lie inside the storage (the checks of reference
-    moonep/api.py:85-97)."""
-    assert pool.is_cuda and pool.ndim >= 2 and pool.shape[0] > 0
-    per_rank = pool[0]
-    assert per_rank.is_contiguous(), "pools must be contiguous within each rank"
-    payload, stride = per_rank.numel(), int(pool.stride(0))
-    assert 0 < payload <= stride, "rank payloads must not overlap"
-    itemsize = pool.element_size()
-    assert 0 < stride * itemsize < (1 << 40) and (stride * itemsize) % 16 == 0
-    assert pool.data_ptr() % 16 == 0, "pools must be 16-byte aligned"
-    last_elem = pool.storage_offset() + stride * (pool.shape[0] - 1) + payload
-    assert last_elem * itemsize <= pool.untyped_storage().nbytes()
+def _rank_stride_of(pool: torch.Tensor, what: str = "pool") -> int:
+    """Elements between two ranks' blocks of an all-rank pool ``[R, ...]``.
+
+    The kernels address rank r's block as ``base + r * stride``; the block itself must be
+    dense.  Blocks may be spaced apart (a caller that carves pools out of a larger arena)
+    as long as they do not overlap, every block starts on a 16-byte boundary and the last
+    one ends inside the storage -- what reference moonep/api.py:85-97 asks of a pool."""
+    assert pool.is_cuda and pool.ndim >= 2 and pool.shape[0] > 0, f"{what}: not an [R, ...] device tensor"
+    block = pool[0]
+    assert block.is_contiguous(), f"{what}: pools must be contiguous within each rank"
+    stride, size, width = int(pool.stride(0)), block.numel(), pool.element_size()
+    assert 0 < size <= stride, f"{what}: rank payloads must not overlap"
+    assert (stride * width) % 16 == 0 and pool.data_ptr() % 16 == 0, \
+        f"{what}: pools must be 16-byte aligned rank by rank"
+    assert stride * width < (1 << 40), f"{what}: rank stride too large"
+    end = pool.storage_offset() + stride * (int(pool.shape[0]) - 1) + size
+    assert end * width <= pool.untyped_storage().nbytes(), f"{what}: last rank's block leaves the storage"
     return stride
+
+
+def _check_local_pool_pairs(what: str, locals_, pools, epn: int, R: int, *, dtypes=None,
+                            fixed_ndim: int | None = 3) -> None:
+    """The (this rank's tensor, all-rank pool) pairs of one operator call.
+
+    Each local tensor is dense ``[epn, ...]`` (exactly ``fixed_ndim`` dimensions when given)
+    of a dtype in ``dtypes``; its pool has the same dtype and device, the shape
+    ``[R, epn, ...]`` with the local tensor's trailing dimensions, and a valid rank stride."""
+    for which, (local, pool) in enumerate(zip(locals_, pools, strict=True)):
+        tag = f"{what}[{which}]"
+        if dtypes is not None:
+            assert local.dtype in dtypes, f"{what}: unsupported weight dtype {local.dtype}"
+        assert local.is_contiguous(), f"{tag}: local tensor must be contiguous"
+        if fixed_ndim is not None:
+            assert local.ndim == fixed_ndim, f"{tag}: local tensor must have {fixed_ndim} dimensions"
+        assert local.ndim >= 2 and int(local.shape[0]) == epn, f"{tag}: local tensor must be [epn={epn}, ...]"
+        assert pool.dtype == local.dtype and pool.device == local.device, \
+            f"{tag}: pool and local tensor differ in dtype or device"
+        assert tuple(pool.shape) == (R, epn, *local.shape[1:]), \
+            f"{tag}: pool must be [R={R}, epn={epn}, {', '.join(str(int(x)) for x in local.shape[1:])}]"
+        _rank_stride_of(pool, tag)
 
 
 def _num_sms_dedup_from_env(max_sms: int) -> int:
@@ -284,6 +313,10 @@ def _create_context(S: int, H: int, K: int, E: int, num_ep_ranks: int, num_sms=N
     assert 0 < N < int32_max, (
         f"planning requires 0 < S*K < int32_max: S={S}, K={K}, S*K={N}, int32_max={int32_max}"
     )
+    # one value past the last slot, R * NvS, marks an entry that nobody copies (an
+    # invalid expert id): it has to be an int32 too
+    assert R * NvS <= int32_max, f"dst encoding requires R*NvS <= int32_max, got {R * NvS}"
+    _lib_init_device()
     if world is None:
         world = EmulatedWorld(S, H, K, E, R, token_padding)
     else:
@@ -298,7 +331,7 @@ def _create_context(S: int, H: int, K: int, E: int, num_ep_ranks: int, num_sms=N
     first_row, first_slot = rank * NvS_padded, rank * mcp + lay["WEIGHTS_OFF"]
     ctx = dict(
         rank=rank, group=group, R=R, E=E, S=S, K=K, H=H, N=N, NvS=NvS, NvS_capacity=N,
-        NvS_padded=NvS_padded, num_sms=num_sms, num_sms_dedup=num_sms_dedup,
+        NvS_padded=NvS_padded, num_sms=num_sms, num_sms_dedup=num_sms_dedup, max_sms=max_sms,
         token_padding=token_padding, token_padding_extra=token_padding_extra, device=device,
         world=world, hidden_buf=world.hidden_buf, meta_buf=world.meta_buf, meta_chunk_padded=mcp,
         hidden_buf_local=world.hidden_buf[first_row: first_row + NvS],
@@ -322,9 +355,13 @@ _LIMITED_LOCK = threading.Lock()
 def _limited_stream(device: int, num_cus: int):
     """(raw handle, torch stream) of THE stream of ``device`` that is bound to
     ``num_cus`` compute units.  One per (device, num_cus), shared by the Buffers
-    that ask for it and kept until the process ends: torch's allocator remembers
-    every stream a tensor was recorded on (``record_stream``) and touches it again
-    when the tensor is freed, so such a stream must never be destroyed."""
+    that ask for it.  The library owns these streams (torch only wraps the handle)
+    and destroys them when the interpreter exits (``_release_limited_streams``): a
+    process that ended with such a queue still open crashed inside a profiler's exit
+    handlers.  For that to be safe no tensor is ever ``record_stream``-ed on them --
+    torch's allocator would touch the stream again when such a tensor is freed,
+    possibly after the stream is gone -- see ``Buffer._on_comm_stream``."""
+    import atexit
     import ctypes
 
     from . import _lib
@@ -335,8 +372,26 @@ def _limited_stream(device: int, num_cus: int):
             with torch.cuda.device(device):
                 _lib.check(_lib.lib().mep_stream_create_limited(num_cus, ctypes.byref(handle)),
                            "mep_stream_create_limited")
+            if not _LIMITED_STREAMS:
+                atexit.register(_release_limited_streams)
             _LIMITED_STREAMS[key] = (handle.value, torch.cuda.ExternalStream(handle.value, device=device))
         return _LIMITED_STREAMS[key]
+
+
+def _release_limited_streams() -> None:
+    """Wait for the device(s) and destroy every CU-masked stream this process made.
+    Runs at interpreter exit; may also be called once no Buffer with ``num_sms`` is in use."""
+    from . import _lib
+    with _LIMITED_LOCK:
+        streams = dict(_LIMITED_STREAMS)
+        _LIMITED_STREAMS.clear()
+    for (device, _), (handle, _) in streams.items():
+        try:
+            with torch.cuda.device(device):
+                torch.cuda.synchronize()
+                _lib.lib().mep_stream_destroy(handle)
+        except Exception:  # noqa: BLE001 - the process is ending; nothing to report to
+            pass
 
 
 class Buffer:
@@ -358,6 +413,7 @@ class Buffer:
         self.enable_pdl = enable_pdl
         self._comm_stream = None
         self._limited_stream = None      # raw handle of a CU-masked comm stream, if any
+        self._inflight = []              # (event, tensors) of asynchronous work on such a stream
         self._destroyed = False
         self._ctx = _create_context(S, H, K, E, num_ep_ranks, num_sms=num_sms,
                                     token_padding=token_padding, group=group, rank=rank,
@@ -403,7 +459,8 @@ class Buffer:
             self._ctx.clear()
         self._ctx = None
         self._comm_stream = None
-        self._limited_stream = None      # the stream itself stays (see _limited_stream)
+        self._limited_stream = None      # the stream itself is shared (see _limited_stream)
+        self._inflight = []              # everything was waited for above
         self._destroyed = True
 
     def __del__(self):
@@ -452,11 +509,21 @@ class Buffer:
         main_stream = torch.cuda.current_stream()
         comm = self._comm_stream
         assert comm is not None, "MoonEP Buffer communication stream is not initialized"
-        self._record_streams(tensors, comm)
+        if self._limited_stream is None:
+            self._record_streams(tensors, comm)
         comm.wait_event(main_stream.record_event())
         with torch.cuda.stream(comm):
             fn()
-            return comm.record_event()
+            done = comm.record_event()
+        if self._limited_stream is not None:
+            # A CU-masked stream is the library's and gets destroyed at exit, so the
+            # allocator must never hold it: instead of record_stream the tensors are kept
+            # alive here until the work on them has finished.  (A synchronous caller's
+            # stream waits for `done` at once, which already orders any reuse.)
+            if not torch.cuda.is_current_stream_capturing():   # events cannot be queried under capture
+                self._inflight = [(ev, ts) for ev, ts in self._inflight if not ev.query()]
+            self._inflight.append((done, [t for t in tensors if t is not None]))
+        return done
 
     def _run_dispatch(self, ctx, hidden_sh, route_weights_sk, planning_args, plan, hidden_nvsh,
                       route_weights_nvs, zero_copy, route_weights_zero_copy, sync) -> None:
@@ -478,8 +545,7 @@ class Buffer:
                     # the reference's count all-gather: my row into every rank's
                     # table; the planner reads the table once all rows are in
                     world.deposit_tokens_per_expert(rank, tpe)
-                    if sync:
-                        world.rendezvous(rank)
+                    world.rendezvous(rank)
                     tpe = world.tpe_table(rank)
                 launch_planning(ctx, topk.reshape(-1), tpe, cu_seqlens, plan, warm=hidden_sh)
                 world.dst_all[rank].copy_(plan.dst)
@@ -524,6 +590,23 @@ class Buffer:
                 "written (or read) their rows: use zero_copy=True, or a world with "
                 "host_threads=True and one thread per rank")
 
+    @staticmethod
+    def _check_count_gather(ctx, tokens_per_expert, sync: bool) -> None:
+        """A per-rank ``tokens_per_expert[E]`` is only a plan input once the other
+        ranks' rows have been gathered beside it.  That happens at a rendezvous of R
+        rank threads; from a single host thread the other rows of the table would be
+        zero or left over from an earlier step and the ranks' plans would disagree
+        (rows of different ranks landing on the same slots)."""
+        R, E = int(ctx["R"]), int(ctx["E"])
+        if R == 1 or tokens_per_expert.numel() != E:
+            return
+        world = ctx["world"]
+        if not (world.host_threads and sync):
+            raise NotImplementedError(
+                "dispatch(tokens_per_expert[E]) of one rank needs the other ranks' counts: pass the "
+                f"gathered tokens_per_expert[R={R}, E={E}], or run every rank on its own host thread "
+                "of an EmulatedWorld(host_threads=True) with inter_rank_sync=True")
+
     # -- public operators ------------------------------------------------------
     def dispatch(self, hidden_sh: torch.Tensor, route_weights_sk=None, topk_experts_sk=None,
                  tokens_per_expert=None, plan: MoonEPCommPlan | None = None,
@@ -560,6 +643,7 @@ class Buffer:
             assert tokens_per_expert.numel() in (int(ctx["E"]), R * int(ctx["E"]))
             assert tokens_per_expert.is_contiguous()
             assert tokens_per_expert.device == hidden_sh.device
+            self._check_count_gather(ctx, tokens_per_expert, bool(inter_rank_sync))
             plan, cu_seqlens = allocate_planning_outputs(ctx)
             planning_args = (topk_experts_sk, tokens_per_expert, cu_seqlens)
         else:
@@ -605,32 +689,17 @@ class Buffer:
         epn = int(ctx["E"]) // R
         local_weights = (local_gate_weight, local_up_weight, local_down_weight)
         pools = (gate_prefetch_buffer, up_prefetch_buffer, down_prefetch_buffer)
-        assert all(t is not None for t in (*local_weights, *pools)), \
-            "prefetch_weight tensors must be provided together"
-        for local, pool in zip(local_weights, pools, strict=True):
-            assert local.dtype in _ELEM_TYPES, \
-                f"prefetch_weight: unsupported weight dtype {local.dtype}"
-            assert local.is_contiguous()
-            assert local.ndim == 3 and int(local.shape[0]) == epn
-            assert pool.dtype == local.dtype and _validate_rank_strided_pool(pool)
-            assert pool.ndim == 4 and tuple(pool.shape[:2]) == (R, epn)
-            assert tuple(pool.shape[2:]) == tuple(local.shape[1:])
-            assert pool.device == local.device
+        assert None not in (*local_weights, *pools), "prefetch_weight tensors must be provided together"
+        _check_local_pool_pairs("prefetch_weight", local_weights, pools, epn, R, dtypes=_ELEM_TYPES)
         local_scales = (local_gate_scale, local_up_scale, local_down_scale)
         scale_pools = (gate_scale_prefetch_buffer, up_scale_prefetch_buffer,
                        down_scale_prefetch_buffer)
+        given = sum(t is not None for t in (*local_scales, *scale_pools))
+        assert given in (0, 6), "prefetch_weight scales must be provided together"
         scales = None
-        if any(t is not None for t in (*local_scales, *scale_pools)):
-            assert all(t is not None for t in (*local_scales, *scale_pools)), \
-                "prefetch_weight scales must be provided together"
-            for local, pool in zip(local_scales, scale_pools, strict=True):
-                assert local.is_contiguous()
-                assert local.ndim >= 2 and int(local.shape[0]) == epn
-                assert pool.dtype == local.dtype and _validate_rank_strided_pool(pool)
-                assert pool.ndim == local.ndim + 1
-                assert tuple(pool.shape[:2]) == (R, epn)
-                assert tuple(pool.shape[2:]) == tuple(local.shape[1:])
-                assert pool.device == local.device
+        if given:
+            _check_local_pool_pairs("prefetch_weight scales", local_scales, scale_pools, epn, R,
+                                    fixed_ndim=None)
             scales = tuple(zip(local_scales, scale_pools, strict=True))
 
         def run():
@@ -689,42 +758,49 @@ class Buffer:
 
     def reduce_grad(self, plan: MoonEPCommPlan | None = None, async_finish: bool = False, *,
                     local_gate_grad=None, local_up_grad=None, local_down_grad=None,
-                    gate_reduce_buffer=None, up_reduce_buffer=None, down_reduce_buffer=None):
+                    gate_reduce_buffer=None, up_reduce_buffer=None, down_reduce_buffer=None,
+                    phase: str = "both"):
         """Sum the weight grads that other ranks accumulated for this rank's
         experts back into its local grads, then zero this rank's own occupied
-        slots (reference moonep/api.py:1121-1208)."""
+        slots (reference moonep/api.py:1121-1208).
+
+        ``phase`` (not in the reference) splits the call where the reference has its
+        cross-rank barrier (moonep/grad_reduce.py:369-372): "reduce" only sums, "clear"
+        only zeroes.  One host thread that plays several ranks on shared pools must run
+        "reduce" for every rank before "clear" for any -- a rank's clear wipes slots that
+        hold *other* ranks' experts -- so "both" is refused there; ranks on the host
+        threads of a ``host_threads`` world meet at a rendezvous between the halves."""
         ctx = self._require_ctx()
         R = int(ctx["R"])
         epn = int(ctx["E"]) // R
         local_grads = (local_gate_grad, local_up_grad, local_down_grad)
         pools = (gate_reduce_buffer, up_reduce_buffer, down_reduce_buffer)
-        assert all(t is not None for t in (*local_grads, *pools)), \
-            "reduce_grad tensors must be provided together"
+        assert None not in (*local_grads, *pools), "reduce_grad tensors must be provided together"
         assert isinstance(plan, MoonEPCommPlan), "Buffer.reduce_grad: plan is required"
-        for local, pool in zip(local_grads, pools, strict=True):
-            assert local.dtype == torch.float32 and local.is_contiguous()
-            assert local.ndim == 3 and int(local.shape[0]) == epn
-            assert pool.dtype == torch.float32 and _validate_rank_strided_pool(pool)
-            assert pool.ndim == 4 and tuple(pool.shape[:2]) == (R, epn)
-            assert tuple(pool.shape[2:]) == tuple(local.shape[1:])
-            assert pool.device == local.device
+        assert phase in ("both", "reduce", "clear"), f"phase must be both, reduce or clear, got {phase!r}"
+        _check_local_pool_pairs("reduce_grad", local_grads, pools, epn, R, dtypes=(torch.float32,))
+        world, rank = ctx["world"], int(ctx["rank"])
+        if phase == "both" and R > 1 and world.attached > 1 and not world.host_threads:
+            raise AssertionError(
+                f"reduce_grad on an EmulatedWorld shared by {world.attached} Buffers driven from one "
+                "host thread: this rank's clear would zero slots that other ranks have not summed "
+                "yet.  Call reduce_grad(..., phase=\"reduce\") for every rank, then "
+                "reduce_grad(..., phase=\"clear\") for every rank, or use a world with "
+                "host_threads=True and one thread per rank")
+
+        def launch(which):
+            for local, pool in zip(local_grads, pools, strict=True):
+                launch_grad_reduce(local, pool, plan.experts_to_copy, rank=rank,
+                                   num_sms=int(ctx["num_sms"]), phase=which)
 
         def run():
-            world, rank = ctx["world"], int(ctx["rank"])
-            if not world.host_threads:
-                for local, pool in zip(local_grads, pools, strict=True):
-                    launch_grad_reduce(local, pool, plan.experts_to_copy, rank=rank,
-                                       num_sms=int(ctx["num_sms"]))
+            if phase != "both" or not world.host_threads:
+                launch(phase)
                 return
-            # ranks on host threads: every rank reads before any rank clears, as the
-            # reference's barrier between the two halves ensures (grad_reduce.py:369-372)
+            # ranks on host threads: every rank reads before any rank clears
             world.rendezvous(rank)
-            for local, pool in zip(local_grads, pools, strict=True):
-                launch_grad_reduce(local, pool, plan.experts_to_copy, rank=rank,
-                                   num_sms=int(ctx["num_sms"]), phase="reduce")
+            launch("reduce")
             world.rendezvous(rank)
-            for local, pool in zip(local_grads, pools, strict=True):
-                launch_grad_reduce(local, pool, plan.experts_to_copy, rank=rank,
-                                   num_sms=int(ctx["num_sms"]), phase="clear")
+            launch("clear")
 
         return self._finish((plan.experts_to_copy, *local_grads, *pools), run, async_finish)

@@ -24,7 +24,7 @@ def launch_combine_prologue(ctx: dict, plan: MoonEPCommPlan, *, pdl_trigger: boo
     """In place on the local shard: primary row <- bf16(fp32 sum of the
     primary and its duplicate rows)."""
     assert isinstance(plan, MoonEPCommPlan)
-    from .dispatch import _require_dedup_map
+    from .dispatch import _require_dedup_map, dup_cu_bound
     _require_dedup_map(ctx, plan, "launch_combine_prologue")
     H, NvS = int(ctx["H"]), int(ctx["NvS"])
     shard = ctx["hidden_buf_local"]
@@ -34,7 +34,7 @@ def launch_combine_prologue(ctx: dict, plan: MoonEPCommPlan, *, pdl_trigger: boo
     assert plan.K <= 32
     rc = _lib.lib().mep_combine_prologue(
         shard.data_ptr(), plan.dup_groups.data_ptr(), plan.dup_loffs.data_ptr(),
-        plan.dup_counts.data_ptr(), NvS, H, _lib.current_stream(),
+        plan.dup_counts.data_ptr(), NvS, H, dup_cu_bound(ctx), _lib.current_stream(),
     )
     _lib.check(rc, "mep_combine_prologue")
 

@@ -4,7 +4,25 @@
 
 #include <vector>
 
-extern "C" int mep_version(void) { return 100; }  // major*10000 + minor*100 + patch
+// major*10000 + minor*100 + patch.  200: mep_grad_reduce takes `flags` before `stream`,
+// mep_dispatch_epilogue / mep_combine_prologue take `max_cus`, mep_init and mep_prefetch_pull exist.
+extern "C" int mep_version(void) { return 200; }
+
+int mep_ensure_init() {
+  static std::atomic<uint64_t> done{0};
+  int dev = 0;
+  MEP_RETURN_IF_HIP(hipGetDevice(&dev));
+  MEP_REQUIRE(dev >= 0 && dev < 64, MEP_ERR_UNSUPPORTED);
+  const uint64_t bit = 1ull << dev;
+  if (done.load(std::memory_order_acquire) & bit) return MEP_OK;
+  int rc = mep_init_planner_kernels();
+  if (rc == MEP_OK) rc = mep_init_stream_kernels();
+  if (rc == MEP_OK) rc = mep_init_gemm_kernels();
+  if (rc == MEP_OK) done.fetch_or(bit, std::memory_order_release);  // racing threads set the same attributes
+  return rc;
+}
+
+extern "C" int mep_init(void) { return mep_ensure_init(); }
 
 extern "C" const char* mep_strerror(int code) {
   switch (code) {

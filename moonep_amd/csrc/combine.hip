@@ -190,6 +190,7 @@ extern "C" int mep_combine(const void* shards, int64_t shard_stride_rows, const 
   MEP_REQUIRE(mode >= MEP_COMBINE_PRIMARIES && mode <= MEP_COMBINE_WEIGHTED, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(mode != MEP_COMBINE_WEIGHTED || wslots, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(K <= 32, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((int64_t)R * NvS <= INT32_MAX, MEP_ERR_UNSUPPORTED);  // raw = R*NvS marks an entry to skip
   MEP_REQUIRE(H % 8 == 0, MEP_ERR_UNSUPPORTED);
   MEP_REQUIRE(shard_stride_rows >= NvS && (!wslots || wslot_stride >= NvS), MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(((uintptr_t)shards % 16 == 0) && ((uintptr_t)out_SH % 16 == 0), MEP_ERR_ALIGNMENT);

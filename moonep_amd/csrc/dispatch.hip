@@ -205,10 +205,15 @@ struct DupArgs {
   int NvS, H;
 };
 
-__global__ __launch_bounds__(kBlock) void epilogue_kernel(DupArgs a) {
+// Workgroups of 4 waves by default; of 16 waves when the caller bounds the number of
+// compute units (one workgroup per CU then, so each CU still has enough rows in flight).
+constexpr int kDupBlockMax = 1024;
+
+__global__ __launch_bounds__(kDupBlockMax) void epilogue_kernel(DupArgs a) {
   const int lane = threadIdx.x & 63;
-  const int gw = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  const int nw = gridDim.x * kWavesPerBlock;
+  const int wpb = blockDim.x >> 6;
+  const int gw = blockIdx.x * wpb + (threadIdx.x >> 6);
+  const int nw = gridDim.x * wpb;
   int ng = a.dup_counts[0];
   if (ng > a.NvS) ng = a.NvS;
   const size_t row_bytes = (size_t)a.H * 2;
@@ -238,10 +243,11 @@ __global__ __launch_bounds__(kBlock) void epilogue_kernel(DupArgs a) {
   }
 }
 
-__global__ __launch_bounds__(kBlock) void prologue_kernel(DupArgs a) {
+__global__ __launch_bounds__(kDupBlockMax) void prologue_kernel(DupArgs a) {
   const int lane = threadIdx.x & 63;
-  const int gw = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  const int nw = gridDim.x * kWavesPerBlock;
+  const int wpb = blockDim.x >> 6;
+  const int gw = blockIdx.x * wpb + (threadIdx.x >> 6);
+  const int nw = gridDim.x * wpb;
   int ng = a.dup_counts[0];
   if (ng > a.NvS) ng = a.NvS;
   const size_t row_bytes = (size_t)a.H * 2;
@@ -272,9 +278,22 @@ __global__ __launch_bounds__(kBlock) void prologue_kernel(DupArgs a) {
   }
 }
 
-int dup_grid(int NvS) {
+// Launch shape of the duplicate kernels (they grid-stride over the groups, whose number is
+// only known on the device).  max_cus <= 0: up to 2048 workgroups of 4 waves.  max_cus = N:
+// at most N workgroups (of 16 waves), so at most N compute units work on it -- the bound
+// the reference sizes these two grids with (MOONEP_NUM_SMS_DEDUP, moonep/api.py:100-120).
+void dup_launch_shape(int NvS, int max_cus, dim3* grid, dim3* block) {
+  if (max_cus > 0) {
+    const int wpb = kDupBlockMax / MEP_WAVE;
+    int blocks = (NvS + wpb - 1) / wpb;
+    if (blocks > max_cus) blocks = max_cus;
+    *grid = dim3(blocks > 0 ? blocks : 1);
+    *block = dim3(kDupBlockMax);
+    return;
+  }
   int blocks = (NvS + kWavesPerBlock - 1) / kWavesPerBlock;
-  return blocks < 2048 ? (blocks > 0 ? blocks : 1) : 2048;
+  *grid = dim3(blocks < 2048 ? (blocks > 0 ? blocks : 1) : 2048);
+  *block = dim3(kBlock);
 }
 
 }  // namespace
@@ -290,6 +309,8 @@ extern "C" int mep_dispatch(const void* hidden_SH, const float* w_SK, const int3
               MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(rank >= 0 && rank < R, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(K <= 32, MEP_ERR_UNSUPPORTED);
+  // an entry decodes as (raw / NvS, raw % NvS); raw = R*NvS (rank R) marks an entry nobody copies
+  MEP_REQUIRE((int64_t)R * NvS <= INT32_MAX, MEP_ERR_UNSUPPORTED);
   MEP_REQUIRE(H % 8 == 0, MEP_ERR_UNSUPPORTED);  // 16-byte row vectors (reference dispatch.py:901)
   MEP_REQUIRE(shard_stride_rows >= NvS && (!wslots || wslot_stride >= NvS), MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(((uintptr_t)hidden_SH % 16 == 0) && ((uintptr_t)shards % 16 == 0), MEP_ERR_ALIGNMENT);
@@ -365,7 +386,7 @@ extern "C" int mep_build_dedup_static(const int32_t* dst_RN, int rank, int S, in
                                       int32_t* dup_counts, void* stream) {
   MEP_REQUIRE(dst_RN && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(S > 0 && K > 0 && R > 0 && NvS > 0 && rank >= 0 && rank < R, MEP_ERR_INVALID_ARG);
-  MEP_REQUIRE((int64_t)S * R < INT32_MAX, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((int64_t)S * R < INT32_MAX && (int64_t)R * NvS <= INT32_MAX, MEP_ERR_UNSUPPORTED);
   MEP_REQUIRE(mep_dedup_scratch_bytes(S, R) <= kStaticDedupBytes, MEP_ERR_STATIC_LIMIT);
   void* p = nullptr;
   const int rc = static_scratch_ptr(&p);
@@ -381,7 +402,7 @@ extern "C" int mep_build_dedup(const int32_t* dst_RN, int rank, int S, int K, in
                                void* workspace, size_t workspace_bytes, void* stream) {
   MEP_REQUIRE(dst_RN && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(S > 0 && K > 0 && R > 0 && NvS > 0 && rank >= 0 && rank < R, MEP_ERR_INVALID_ARG);
-  MEP_REQUIRE((int64_t)S * R < INT32_MAX, MEP_ERR_UNSUPPORTED);
+  MEP_REQUIRE((int64_t)S * R < INT32_MAX && (int64_t)R * NvS <= INT32_MAX, MEP_ERR_UNSUPPORTED);
   MEP_REQUIRE(workspace && workspace_bytes >= mep_dedup_scratch_bytes(S, R), MEP_ERR_SCRATCH);
   DedupArgs a;
   a.dst = dst_RN; a.dup_groups = dup_groups; a.dup_loffs = dup_loffs; a.dup_counts = dup_counts;
@@ -399,24 +420,28 @@ extern "C" int mep_build_dedup(const int32_t* dst_RN, int rank, int S, int K, in
 
 extern "C" int mep_dispatch_epilogue(void* shard, const int32_t* dup_groups,
                                      const int32_t* dup_loffs, const int32_t* dup_counts, int NvS,
-                                     int H, void* stream) {
+                                     int H, int max_cus, void* stream) {
   MEP_REQUIRE(shard && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(NvS > 0 && H > 0, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(H % 8 == 0, MEP_ERR_UNSUPPORTED);
   MEP_REQUIRE((uintptr_t)shard % 16 == 0, MEP_ERR_ALIGNMENT);
   DupArgs a{(uint16_t*)shard, dup_groups, dup_loffs, dup_counts, NvS, H};
-  hipLaunchKernelGGL(epilogue_kernel, dim3(dup_grid(NvS)), dim3(kBlock), 0, (hipStream_t)stream, a);
+  dim3 grid, block;
+  dup_launch_shape(NvS, max_cus, &grid, &block);
+  hipLaunchKernelGGL(epilogue_kernel, grid, block, 0, (hipStream_t)stream, a);
   return mep_launch_status();
 }
 
 extern "C" int mep_combine_prologue(void* shard, const int32_t* dup_groups,
                                     const int32_t* dup_loffs, const int32_t* dup_counts, int NvS,
-                                    int H, void* stream) {
+                                    int H, int max_cus, void* stream) {
   MEP_REQUIRE(shard && dup_groups && dup_loffs && dup_counts, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(NvS > 0 && H > 0, MEP_ERR_INVALID_ARG);
   MEP_REQUIRE(H % 8 == 0, MEP_ERR_UNSUPPORTED);
   MEP_REQUIRE((uintptr_t)shard % 16 == 0, MEP_ERR_ALIGNMENT);
   DupArgs a{(uint16_t*)shard, dup_groups, dup_loffs, dup_counts, NvS, H};
-  hipLaunchKernelGGL(prologue_kernel, dim3(dup_grid(NvS)), dim3(kBlock), 0, (hipStream_t)stream, a);
+  dim3 grid, block;
+  dup_launch_shape(NvS, max_cus, &grid, &block);
+  hipLaunchKernelGGL(prologue_kernel, grid, block, 0, (hipStream_t)stream, a);
   return mep_launch_status();
 }

@@ -25,17 +25,6 @@
 // (one L2) work on the same 8 row tiles and neighbouring weight tiles.
 #include "mep_common.h"
 
-// MEP_GEMM_PROBE (tests/host/gemm_clock_probe only; never defined in the library build):
-// 1 = the kernel as it is, 2 = no global loads (consumers alone), 3 = no LDS reads or MFMAs
-// (producers alone); every tile adds its core clocks and its constant-rate wall ticks to
-// g_gemm_probe, which tells the clock the chip sustains under each of the three.
-#ifndef MEP_GEMM_PROBE
-#define MEP_GEMM_PROBE 0
-#endif
-#if MEP_GEMM_PROBE
-__device__ unsigned long long g_gemm_probe[4];  // core clocks, wall ticks, tiles
-#endif
-
 #include <atomic>
 
 namespace {
@@ -119,9 +108,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
   static_assert(kProducers == 2, "the lane offsets of the pieces assume that a producer wave's pieces share a parity");
   extern __shared__ __attribute__((aligned(1024))) char gsm[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-#if MEP_GEMM_PROBE
-  const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
-#endif
 
   // ---- which tile.  XCD x (workgroups x, x+8, ...) walks a contiguous eighth of
   // the tile list, in launch order, so the tiles that run on an XCD at one time
@@ -246,13 +232,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
         else if (BKN) src = pb0 + (size_t)(k0 + 2 * (j - kBM / 8)) * a.N;
         else if (j < kBM / 8 + kBN / 16) src = pb0 + (size_t)(8 * (j - kBM / 8)) * K + k0;
         else src = pb1 + (size_t)(8 * (j - kBM / 8 - kBN / 16)) * K + k0;
-#if MEP_GEMM_PROBE == 2
-        (void)src; (void)base;
-#else
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                          (__attribute__((address_space(3))) void*)(base + j * 1024),
                                          16, 0, 0);
-#endif
       }
     };
     const int klast = (KT - 1) * kBK;
@@ -306,9 +288,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
     const char* sb = gsm + st * kStage;
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
-#if MEP_GEMM_PROBE == 3
-      continue;
-#endif
       const int col = ((2 * ks + half) ^ sw) * 16;
       const mep_bf16x8 a0 = *(const mep_bf16x8*)(sb + oa0 + col);
       const mep_bf16x8 a1 = *(const mep_bf16x8*)(sb + oa1 + col);
@@ -332,13 +311,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void grouped_gemm_nt_kernel(GemmAr
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   }
 
-#if MEP_GEMM_PROBE
-  if (tid == 0) {
-    atomicAdd(&g_gemm_probe[0], (unsigned long long)(clock64() - probe_c0));
-    atomicAdd(&g_gemm_probe[1], (unsigned long long)(wall_clock64() - probe_w0));
-    atomicAdd(&g_gemm_probe[2], 1ull);
-  }
-#endif
   // ---- epilogue.  acc[i][j][v]: row 64*wm + 32*i + 8*(v/4) + 4*(lane/32) + v%4,
   // column (lane % 32) of the j-th 32-wide block
   const int ldc = a.N;
@@ -402,9 +374,6 @@ __global__ __launch_bounds__(kT2Threads, 1) void grouped_gemm256_kernel(GemmArgs
   static_assert(!BKN || !SWIGLU, "[K, N] weights: plain and dual products only");
   extern __shared__ __attribute__((aligned(1024))) char gsm[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-#if MEP_GEMM_PROBE
-  const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
-#endif
 
   // ---- tile list: group g has (h + 1) / 2 row tiles, h = its 128-row blocks
   int total_rt = 0;
@@ -495,12 +464,8 @@ __global__ __launch_bounds__(kT2Threads, 1) void grouped_gemm256_kernel(GemmArgs
     char* base = gsm + stage * kT2Stage + wave * 8 * 1024;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-#if MEP_GEMM_PROBE == 2
-      (void)base; (void)off;
-#else
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[q] + off),
                                        (__attribute__((address_space(3))) void*)(base + q * 1024), 16, 0, 0);
-#endif
     }
   };
 
@@ -537,9 +502,6 @@ __global__ __launch_bounds__(kT2Threads, 1) void grouped_gemm256_kernel(GemmArgs
     if (works) {
 #pragma unroll
       for (int ks = 0; ks < kBK / 16; ++ks) {
-#if MEP_GEMM_PROBE == 3
-        continue;
-#endif
         const int col = ((2 * ks + half) ^ sw) * 16;
         mep_bf16x8 fa[4], fb[2];
 #pragma unroll
@@ -564,13 +526,6 @@ __global__ __launch_bounds__(kT2Threads, 1) void grouped_gemm256_kernel(GemmArgs
     __builtin_amdgcn_s_barrier();  // ... for everyone, and everyone is done with this one
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   }
-#if MEP_GEMM_PROBE
-  if (tid == 0) {
-    atomicAdd(&g_gemm_probe[0], (unsigned long long)(clock64() - probe_c0));
-    atomicAdd(&g_gemm_probe[1], (unsigned long long)(wall_clock64() - probe_w0));
-    atomicAdd(&g_gemm_probe[2], 1ull);
-  }
-#endif
   if (!works) return;
 
   // ---- epilogue.  acc[i][j][v]: row 128 wm + 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,
@@ -881,20 +836,13 @@ int gemm256_launch(const GemmArgs& a0, hipStream_t st) {
   MEP_REQUIRE(total > 0 && total < (1 << 30), MEP_ERR_UNSUPPORTED);
   const int per_xcd = (int)((total + 7) / 8);
   const size_t lds = 2 * (size_t)kT2Stage;
-  static std::atomic<uint64_t> opted{0};
-  int dev = 0;
-  MEP_RETURN_IF_HIP(hipGetDevice(&dev));
-  const uint64_t bit = 1ull << (dev & 63);
-  if (!(opted.load(std::memory_order_acquire) & bit)) {
-    MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)grouped_gemm256_kernel<MODE, BKN>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    opted.fetch_or(bit, std::memory_order_release);
-  }
+  const int irc = mep_ensure_init();  // the LDS opt-in of this kernel, once per device
+  if (irc != MEP_OK) return irc;
   hipLaunchKernelGGL((grouped_gemm256_kernel<MODE, BKN>), dim3(per_xcd * 8), dim3(kT2Threads), lds, st, a);
   return mep_launch_status();
 }
 
-// 144 KB of dynamic LDS needs the opt-in, once per device and kernel
+// 144 KB of dynamic LDS: opted in by mep_init_gemm_kernels
 template <int MODE, bool BKN = false>
 int gemm_launch(const GemmArgs& a0, int64_t total, hipStream_t st) {
   GemmArgs a = a0;
@@ -902,17 +850,8 @@ int gemm_launch(const GemmArgs& a0, int64_t total, hipStream_t st) {
   MEP_REQUIRE(total > 0 && total < (1 << 30), MEP_ERR_UNSUPPORTED);
   const int per_xcd = (int)((total + 7) / 8);
   const size_t lds = (size_t)kStages * kStage;
-  static std::atomic<uint64_t> opted{0};
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return (int)e;
-  const uint64_t bit = 1ull << (dev & 63);
-  if (!(opted.load(std::memory_order_acquire) & bit)) {
-    e = hipFuncSetAttribute((const void*)grouped_gemm_nt_kernel<MODE, BKN>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    opted.fetch_or(bit, std::memory_order_release);
-  }
+  const int irc = mep_ensure_init();
+  if (irc != MEP_OK) return irc;
   hipLaunchKernelGGL((grouped_gemm_nt_kernel<MODE, BKN>), dim3(per_xcd * 8), dim3(kGemmThreads), lds, st, a);
   return mep_launch_status();
 }
@@ -930,15 +869,8 @@ int wgrad256_launch(const GemmArgs& a, hipStream_t st) {
   const int64_t per_xcd = (int64_t)per_pair * (a.G / 2);
   MEP_REQUIRE(per_xcd > 0 && per_xcd < (1 << 27), MEP_ERR_UNSUPPORTED);
   const size_t lds = 2 * (size_t)kW2Stage;
-  static std::atomic<uint64_t> opted{0};
-  int dev = 0;
-  MEP_RETURN_IF_HIP(hipGetDevice(&dev));
-  const uint64_t bit = 1ull << (dev & 63);
-  if (!(opted.load(std::memory_order_acquire) & bit)) {
-    MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)wgrad256_kernel<TN>,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    opted.fetch_or(bit, std::memory_order_release);
-  }
+  const int irc = mep_ensure_init();
+  if (irc != MEP_OK) return irc;
   hipLaunchKernelGGL(wgrad256_kernel<TN>, dim3((unsigned)(per_xcd * 8)), dim3(kW2Threads), lds, st, a, map);
   return mep_launch_status();
 }
@@ -969,12 +901,12 @@ GemmArgs nt_args(const void* A, const void* B, const void* B2, const int32_t* cu
 // the CUs.  Measured at 34 688 rows, H = 7168, H' = 2048: 5-8 % faster where a launch has at
 // least eight of them per CU (SwiGLU, down, the dual input gradient), 12 % slower at five
 // (dy * down, 2048 output columns).
-// MEP_GEMM_ROW_TILE=128 or 256 in the environment forces one (tests run both on small shapes).
+// mep_set_gemm_row_tile(128 or 256) forces one (tests run both on small shapes).
+std::atomic<int> g_forced_row_tile{0};
+
 static bool use_256_row_tiles(const GemmArgs& a) {
-  if (const char* e = getenv("MEP_GEMM_ROW_TILE")) {
-    if (e[0] == '2') return true;
-    if (e[0] == '1') return false;
-  }
+  const int forced = g_forced_row_tile.load(std::memory_order_relaxed);
+  if (forced) return forced == 256;
   const int cus = mep_device_cu_count();
   return (int64_t)(a.M / kT2Rows) * a.ntiles >= 8 * (int64_t)(cus > 0 ? cus : 256);
 }
@@ -1001,19 +933,44 @@ int gemm_nt_forward(const void* A, const void* B, const void* B_up, const int32_
                 : gemm_launch<kModeScale>(a, total, (hipStream_t)stream);
 }
 
+template <class Kern>
+int opt_in_lds(Kern kern, size_t bytes) {
+  MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)bytes));
+  return MEP_OK;
+}
+
 }  // namespace
 
-#if MEP_GEMM_PROBE
-extern "C" int mep_gemm_probe_read(unsigned long long* out3, int reset) {
-  hipError_t e = hipMemcpyFromSymbol(out3, HIP_SYMBOL(g_gemm_probe), 3 * sizeof(unsigned long long));
-  if (e != hipSuccess) return (int)e;
-  if (reset) {
-    const unsigned long long z[3] = {0, 0, 0};
-    e = hipMemcpyToSymbol(HIP_SYMBOL(g_gemm_probe), z, sizeof(z));
-  }
-  return (int)e;
+// Every GEMM kernel uses more dynamic LDS than a kernel gets without asking: the opt-ins
+// for the current device, made once from mep_init (never from a launch, which may be
+// under stream capture).
+int mep_init_gemm_kernels() {
+  const size_t ring = (size_t)kStages * kStage, two = 2 * (size_t)kT2Stage, w2 = 2 * (size_t)kW2Stage;
+  int rc = MEP_OK;
+#define MEP_OPT(k, b) if (rc == MEP_OK) rc = opt_in_lds(k, b)
+  MEP_OPT((grouped_gemm_nt_kernel<kModeScale, false>), ring);
+  MEP_OPT((grouped_gemm_nt_kernel<kModeSwiglu, false>), ring);
+  MEP_OPT((grouped_gemm_nt_kernel<kModeDual, false>), ring);
+  MEP_OPT((grouped_gemm_nt_kernel<kModeWgrad, false>), ring);
+  MEP_OPT((grouped_gemm_nt_kernel<kModeScale, true>), ring);
+  MEP_OPT((grouped_gemm_nt_kernel<kModeDual, true>), ring);
+  MEP_OPT((grouped_gemm256_kernel<kModeScale, false>), two);
+  MEP_OPT((grouped_gemm256_kernel<kModeSwiglu, false>), two);
+  MEP_OPT((grouped_gemm256_kernel<kModeDual, false>), two);
+  MEP_OPT((grouped_gemm256_kernel<kModeScale, true>), two);
+  MEP_OPT((grouped_gemm256_kernel<kModeDual, true>), two);
+  MEP_OPT(wgrad256_kernel<false>, w2);
+  MEP_OPT(wgrad256_kernel<true>, w2);
+#undef MEP_OPT
+  return rc;
 }
-#endif
+
+extern "C" int mep_set_gemm_row_tile(int rows) {
+  MEP_REQUIRE(rows == 0 || rows == 128 || rows == 256, MEP_ERR_INVALID_ARG);
+  g_forced_row_tile.store(rows, std::memory_order_relaxed);
+  return MEP_OK;
+}
 
 extern "C" int mep_grouped_gemm_nt(const void* A, const void* B, const void* B_up,
                                    const int32_t* cu_seqlens, int G, void* C,

@@ -29,6 +29,16 @@ static inline int mep_launch_status() {
   return e == hipSuccess ? MEP_OK : (int)e;
 }
 
+// Kernels that use more dynamic LDS than the 64 KB a kernel gets without asking must be
+// opted in with hipFuncSetAttribute, per device, and not from inside a stream capture.
+// Each source file opts its own kernels in for the current device; mep_ensure_init runs all
+// of them once per device (mep_init() is its exported name).  Launch sites of such kernels
+// call it too, so a device that nobody initialised still works outside capture.
+int mep_init_planner_kernels();
+int mep_init_stream_kernels();
+int mep_init_gemm_kernels();
+int mep_ensure_init();
+
 // CUs of the current device, asked once per device (-1 when the runtime cannot tell)
 static inline int mep_device_cu_count() {
   static std::atomic<int> cached[64];

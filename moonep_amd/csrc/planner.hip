@@ -340,7 +340,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   // An entry with an invalid expert id gets destination rank R: dispatch and
   // combine skip such entries (they never write or read outside the R shards),
   // the duplicate-group builder matches no rank to it.
-  int dv = (int)min((int64_t)R * NvS, (int64_t)INT32_MAX), dest = -1;
+  int dv = R * NvS, dest = -1;  // fits: the host requires R*NvS <= INT32_MAX
   if (e >= 0) {
     dest = 0;
     int before = 0;
@@ -487,19 +487,9 @@ int plan_launch(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int n
   } else if (c.lds_tables) {
     hipLaunchKernelGGL((plan_kernel<256, true>), grid, dim3(256), c.lds_bytes, st, a);
   } else {
-    if (c.opt_in) {
-      // once per device: later launches (also under stream capture) find it set
-      static std::atomic<uint64_t> opted{0};
-      int dev = 0;
-      hipError_t e = hipGetDevice(&dev);
-      if (e != hipSuccess) return (int)e;
-      const uint64_t bit = 1ull << (dev & 63);
-      if (!(opted.load(std::memory_order_acquire) & bit)) {
-        e = hipFuncSetAttribute((const void*)plan_kernel<256, false>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsOptInLimit);
-        if (e != hipSuccess) return (int)e;
-        opted.fetch_or(bit, std::memory_order_release);
-      }
+    if (c.opt_in) {  // more dynamic LDS than the default limit: opted in by mep_init_planner_kernels
+      const int irc = mep_ensure_init();
+      if (irc != MEP_OK) return irc;
     }
     hipLaunchKernelGGL((plan_kernel<256, false>), grid, dim3(256), c.lds_bytes, st, a);
   }
@@ -507,6 +497,13 @@ int plan_launch(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int n
 }
 
 }  // namespace
+
+// LDS opt-in of the planner variant for very large expert counts, for the current device
+int mep_init_planner_kernels() {
+  MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)plan_kernel<256, false>,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsOptInLimit));
+  return MEP_OK;
+}
 
 extern "C" int mep_plan_ranks(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int nranks,
                               int S, int K, int E, int R, int token_padding, int NvS, int32_t* dst,

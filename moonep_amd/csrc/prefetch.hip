@@ -15,6 +15,7 @@
 namespace {
 
 constexpr int kBlock = 256;
+constexpr size_t kReduceLdsMax = 150 * 1024;  // dynamic LDS the slot reduction may ask for
 constexpr int kVecPerThread = 4;                       // 16-byte vectors in flight per thread
 constexpr int kTileBytes = kBlock * kVecPerThread * 16;  // 16 KiB per workgroup step
 constexpr int kMaxTensors = 6;
@@ -223,6 +224,105 @@ __global__ __launch_bounds__(kBlock) void prefetch_kernel(PrefetchArgs a) {
     const unsigned wn = w + gridDim.x;
     const bool more = wn < total && wn > w;  // workgroup-uniform
     PrefetchTile nx = cur;
+    mep_u4 nv[kVecPerThread] = {};
+    if (more) { nx = decode(wn); load(nx, nv); }
+    store(cur, v);
+    if (!more) break;
+    cur = nx; w = wn;
+#pragma unroll
+    for (int i = 0; i < kVecPerThread; ++i) v[i] = nv[i];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// pull view of the prefetch: ONE rank's slots filled from all owners
+// ---------------------------------------------------------------------------
+struct PullArgs {
+  const char* owners[kMaxTensors];    // expert e of owner o at owners + o*owner_stride + (e % epn)*bytes
+  char* pool[kMaxTensors];
+  int64_t owner_stride[kMaxTensors];  // bytes
+  int64_t rank_stride[kMaxTensors];   // bytes
+  SpreadTiles st[kMaxTensors];
+  const int* etc;
+  int ntensors, rank, epn, R;
+};
+
+// The occupied slots of `rank` form the work list (slot b <- expert etc[rank, b]); persistent
+// workgroups walk (tensor, occupied slot, tile) in the tile layout of the push kernel, the
+// next tile's loads issued before the current tile's stores.  LDS: slot[epn], expert[epn], n.
+__global__ __launch_bounds__(kBlock) void prefetch_pull_kernel(PullArgs a) {
+  extern __shared__ int smem[];
+  int* s_slot = smem;
+  int* s_exp = smem + a.epn;
+  int* s_n = s_exp + a.epn;
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    int n = 0;
+    for (int c = 0; c < a.epn; c += 64) {
+      const int b = c + lane;
+      const int e = b < a.epn ? a.etc[a.rank * a.epn + b] : -1;
+      const bool ok = e >= 0 && e < a.R * a.epn;
+      const uint64_t m = __ballot(ok);
+      if (ok) {
+        const int i = n + __popcll(m & mep_lanes_lt());
+        s_slot[i] = b; s_exp[i] = e;
+      }
+      n += __popcll(m);
+    }
+    if (lane == 0) *s_n = n;
+  }
+  __syncthreads();
+  const unsigned n_slots = (unsigned)__builtin_amdgcn_readfirstlane(*s_n);
+  if (n_slots == 0) return;
+  unsigned total = 0;
+  for (int ti = 0; ti < a.ntensors; ++ti) total += (unsigned)a.st[ti].tiles * n_slots;
+  struct Tile { int ti, b, e, step; int64_t off; bool whole; };
+  auto decode = [&](unsigned w) {
+    Tile p;
+    p.ti = 0;
+    unsigned per = (unsigned)a.st[0].tiles;
+    while (w >= per * n_slots) { w -= per * n_slots; per = (unsigned)a.st[++p.ti].tiles; }
+    const unsigned si = w / per, tile = w - si * per;
+    p.b = __builtin_amdgcn_readfirstlane(s_slot[si]);
+    p.e = __builtin_amdgcn_readfirstlane(s_exp[si]);
+    p.off = a.st[p.ti].first(tile, &p.step);
+    p.whole = a.st[p.ti].whole(tile);
+    return p;
+  };
+  auto load = [&](const Tile& p, mep_u4* v) {
+    const int64_t bytes = a.st[p.ti].bytes;
+    const int o = p.e / a.epn, le = p.e - o * a.epn;
+    const char* src = a.owners[p.ti] + (int64_t)o * a.owner_stride[p.ti] + (int64_t)le * bytes + p.off;
+    if (p.whole) {
+#pragma unroll
+      for (int i = 0; i < kVecPerThread; ++i) v[i] = mep_ld16_stream(src + (int64_t)i * p.step);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kVecPerThread; ++i)
+        if (p.off + (int64_t)i * p.step < bytes) v[i] = mep_ld16_stream(src + (int64_t)i * p.step);
+    }
+  };
+  auto store = [&](const Tile& p, const mep_u4* v) {
+    const int64_t bytes = a.st[p.ti].bytes;
+    char* dst = a.pool[p.ti] + (int64_t)a.rank * a.rank_stride[p.ti] + (int64_t)p.b * bytes + p.off;
+    if (p.whole) {
+#pragma unroll
+      for (int i = 0; i < kVecPerThread; ++i) mep_st16_through(dst + (int64_t)i * p.step, v[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kVecPerThread; ++i)
+        if (p.off + (int64_t)i * p.step < bytes) mep_st16_through(dst + (int64_t)i * p.step, v[i]);
+    }
+  };
+  unsigned w = blockIdx.x;
+  if (w >= total) return;
+  Tile cur = decode(w);
+  mep_u4 v[kVecPerThread] = {};
+  load(cur, v);
+  for (;;) {
+    const unsigned wn = w + gridDim.x;
+    const bool more = wn < total && wn > w;  // workgroup-uniform
+    Tile nx = cur;
     mep_u4 nv[kVecPerThread] = {};
     if (more) { nx = decode(wn); load(nx, nv); }
     store(cur, v);
@@ -480,6 +580,51 @@ extern "C" int mep_prefetch(int ntensors, const void* const* local, void* const*
   return mep_launch_status();
 }
 
+extern "C" int mep_prefetch_pull(int ntensors, const void* const* owners,
+                                 const int64_t* owner_stride_bytes, void* const* pool,
+                                 const int64_t* rank_stride_bytes, const int64_t* bytes_per_expert,
+                                 const int32_t* experts_to_copy, int rank, int epn, int R,
+                                 void* stream) {
+  MEP_REQUIRE(owners && owner_stride_bytes && pool && rank_stride_bytes && bytes_per_expert &&
+                  experts_to_copy, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(ntensors > 0 && ntensors <= kMaxTensors, MEP_ERR_INVALID_ARG);
+  MEP_REQUIRE(epn > 0 && R > 0 && rank >= 0 && rank < R, MEP_ERR_INVALID_ARG);
+  const size_t lds = (2 * (size_t)epn + 1) * sizeof(int);
+  MEP_REQUIRE(lds <= 64 * 1024, MEP_ERR_UNSUPPORTED);
+  PullArgs a;
+  a.ntensors = ntensors; a.rank = rank; a.epn = epn; a.R = R; a.etc = experts_to_copy;
+  int64_t all_tiles = 0;
+  for (int i = 0; i < ntensors; ++i) {
+    MEP_REQUIRE(owners[i] && pool[i], MEP_ERR_INVALID_ARG);
+    MEP_REQUIRE(bytes_per_expert[i] > 0 && bytes_per_expert[i] % 16 == 0, MEP_ERR_UNSUPPORTED);
+    MEP_REQUIRE(rank_stride_bytes[i] >= bytes_per_expert[i] * epn &&
+                    owner_stride_bytes[i] >= bytes_per_expert[i] * epn, MEP_ERR_INVALID_ARG);
+    MEP_REQUIRE(rank_stride_bytes[i] % 16 == 0 && owner_stride_bytes[i] % 16 == 0 &&
+                    (uintptr_t)owners[i] % 16 == 0 && (uintptr_t)pool[i] % 16 == 0, MEP_ERR_ALIGNMENT);
+    a.owners[i] = (const char*)owners[i]; a.pool[i] = (char*)pool[i];
+    a.owner_stride[i] = owner_stride_bytes[i]; a.rank_stride[i] = rank_stride_bytes[i];
+    a.st[i] = SpreadTiles(bytes_per_expert[i]);
+    all_tiles += a.st[i].tiles;
+  }
+  for (int i = ntensors; i < kMaxTensors; ++i) {
+    a.owners[i] = nullptr; a.pool[i] = nullptr; a.owner_stride[i] = 0; a.rank_stride[i] = 0;
+    a.st[i] = SpreadTiles(0);
+  }
+  MEP_REQUIRE(all_tiles * epn < ((int64_t)1 << 31), MEP_ERR_UNSUPPORTED);
+  const int cus = mep_device_cu_count();
+  int64_t blocks = 2 * (int64_t)(cus > 0 ? cus : 256);
+  if (all_tiles * epn < blocks) blocks = all_tiles * epn;
+  hipLaunchKernelGGL(prefetch_pull_kernel, dim3((unsigned)blocks), dim3(kBlock), lds, (hipStream_t)stream, a);
+  return mep_launch_status();
+}
+
+// LDS opt-in of the slot reduction for large rank x slot tables, for the current device
+int mep_init_stream_kernels() {
+  MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)grad_reduce_kernel,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kReduceLdsMax));
+  return MEP_OK;
+}
+
 extern "C" int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t rank_stride_elems,
                                const int32_t* experts_to_copy, int rank, int epn, int R,
                                int64_t elems_per_expert, unsigned flags, void* stream) {
@@ -494,10 +639,11 @@ extern "C" int mep_grad_reduce(float* local_grad, float* reduce_pool, int64_t ra
   // slot table + own foreign-held slots + a pool offset per list entry
   const size_t lds = slot_table_bytes(R, epn) + ((size_t)epn + 2) * sizeof(int) +
                      (size_t)R * epn * sizeof(int64_t) + 8;
-  MEP_REQUIRE(lds <= 150 * 1024, MEP_ERR_UNSUPPORTED);
-  if (lds > 64 * 1024)  // large rank x slot tables: more dynamic LDS than the default limit
-    MEP_RETURN_IF_HIP(hipFuncSetAttribute((const void*)grad_reduce_kernel,
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  MEP_REQUIRE(lds <= kReduceLdsMax, MEP_ERR_UNSUPPORTED);
+  if (lds > 64 * 1024) {  // large rank x slot tables: opted in by mep_init_stream_kernels
+    const int irc = mep_ensure_init();
+    if (irc != MEP_OK) return irc;
+  }
   ReduceArgs a{local_grad, reduce_pool, rank_stride_elems, elems_per_expert, experts_to_copy,
                rank, epn, R, flags};
   const SpreadTiles rt(elems_per_expert * 4);

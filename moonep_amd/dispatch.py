@@ -112,6 +112,15 @@ def launch_build_dedup(ctx: dict, dst_all_ranks: torch.Tensor, plan: MoonEPCommP
     _lib.check(rc, "mep_build_dedup")
 
 
+def dup_cu_bound(ctx: dict) -> int:
+    """Compute units the standalone duplicate kernels may use: the context's
+    ``num_sms_dedup`` (``MOONEP_NUM_SMS_DEDUP``, reference moonep/api.py:100-120) when it
+    is below the device's CU count, else 0 = no bound (the kernels then pick the grid that
+    fills the GPU)."""
+    n, all_cus = int(ctx.get("num_sms_dedup", 0) or 0), int(ctx.get("max_sms", 0) or 0)
+    return n if 0 < n < all_cus else 0
+
+
 def launch_dispatch_epilogue(ctx: dict, plan: MoonEPCommPlan, *, pdl_launch: bool = False) -> None:
     """Copy every primary row of the local shard to its duplicate rows."""
     assert isinstance(plan, MoonEPCommPlan)
@@ -120,6 +129,7 @@ def launch_dispatch_epilogue(ctx: dict, plan: MoonEPCommPlan, *, pdl_launch: boo
     assert shard.dtype == torch.bfloat16 and shard.is_contiguous()
     rc = _lib.lib().mep_dispatch_epilogue(
         shard.data_ptr(), plan.dup_groups.data_ptr(), plan.dup_loffs.data_ptr(),
-        plan.dup_counts.data_ptr(), int(ctx["NvS"]), int(ctx["H"]), _lib.current_stream(),
+        plan.dup_counts.data_ptr(), int(ctx["NvS"]), int(ctx["H"]), dup_cu_bound(ctx),
+        _lib.current_stream(),
     )
     _lib.check(rc, "mep_dispatch_epilogue")

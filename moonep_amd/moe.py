@@ -13,12 +13,11 @@ shared ``EmulatedWorld``): every rank dispatches before any rank's experts
 run, every rank's experts finish before any rank combines -- the ordering the
 reference gets from its cross-rank barriers.
 
-``grouped_ffn`` is a plain PyTorch consumer (library GEMMs per group, group
-bounds read on the host) meant for parity tests; ``group_expert_ffn_hip`` is the
-same layer stage on the matrix cores, forward and backward: prefetch of the
-compute views, the grouped SwiGLU FFN of every rank, and in backward the grouped
-input / weight gradient GEMMs followed by ``reduce_grad`` in fp32 -- no PyTorch
-GEMM on either pass.
+``group_expert_ffn_hip`` is the expert stage of the layer on the matrix cores,
+forward and backward: the compute views of every rank (its local experts, then
+its prefetch slots filled by one ``launch_prefetch_pull``), the grouped SwiGLU FFN
+of every rank, and in backward the grouped input / weight gradient GEMMs followed
+by ``reduce_grad`` in fp32 -- no PyTorch GEMM on either pass.
 """
 
 from __future__ import annotations
@@ -28,7 +27,7 @@ import torch
 from . import ffn
 from .api import Buffer, EmulatedWorld
 from .grad_reduce import launch_grad_reduce
-from .prefetch import launch_prefetch
+from .prefetch import launch_prefetch_pull
 
 
 class EmulatedGroup:
@@ -130,8 +129,8 @@ class _GroupPrefetch(torch.autograd.Function):
         R, epn = group.R, group.epn
         local = master.to(torch.bfloat16).contiguous()
         pool = torch.zeros_like(local)
-        for r in range(R):
-            launch_prefetch((local[r],) * 3, (pool,) * 3, experts_to_copy, rank=r)
+        for r in range(R):     # a rank's slots filled from all owners in one launch
+            launch_prefetch_pull((local,) * 3, (pool,) * 3, experts_to_copy, rank=r)
         ctx.group, ctx.etc = group, experts_to_copy
         return torch.cat([local, pool], dim=1)
 
@@ -153,7 +152,7 @@ class _GroupExpertFFN(torch.autograd.Function):
 
     fp32 master weights in the orientation the kernels read: gate / up
     [R, epn, H', H], down [R, epn, H, H'].  Forward: bf16 compute views (local
-    experts, then the prefetch slots filled by ``launch_prefetch``), then per rank
+    experts, then the prefetch slots filled by ``launch_prefetch_pull``), then per rank
     the fused gate/up GEMM and the down GEMM with the route weight applied.
     Backward: the grouped gradient GEMMs per rank, then ``launch_grad_reduce``
     sums every slot's fp32 weight gradient into its owner's."""
@@ -163,8 +162,8 @@ class _GroupExpertFFN(torch.autograd.Function):
         R, tp = group.R, group.world.token_padding
         local = [m.detach().to(torch.bfloat16).contiguous() for m in (gate_m, up_m, down_m)]
         pools = [torch.zeros_like(t) for t in local]
-        for r in range(R):
-            launch_prefetch(tuple(t[r] for t in local), tuple(pools), experts_to_copy, rank=r)
+        for r in range(R):     # a rank's slots filled from all owners in one launch
+            launch_prefetch_pull(tuple(local), tuple(pools), experts_to_copy, rank=r)
         views = [torch.cat([l, p], dim=1) for l, p in zip(local, pools)]      # [R, 2*epn, ...]
         outs, saved = [], []
         for r in range(R):
@@ -223,24 +222,3 @@ def group_combine(group, plans, y_all):
 
 def group_compute_views(group, experts_to_copy, master_weights):
     return _GroupPrefetch.apply(group, experts_to_copy, master_weights)
-
-
-def grouped_ffn(rows, slots, cu_seqlens, gate, up, down):
-    """Reference consumer of one rank's dispatched rows.
-
-    rows [NvS,H] bf16, slots [NvS] fp32 route weights, cu_seqlens [2*epn]
-    (padded end offset of every group), gate/up/down [2*epn,H,H'] compute
-    views.  Group g applies ``w * (silu(x @ gate[g]) * (x @ up[g])) @ down[g].T``
-    to its rows; rows outside every group are zero.
-    """
-    out = torch.zeros_like(rows)
-    ends = cu_seqlens.tolist()
-    start = 0
-    for g, end in enumerate(ends):
-        if end > start:
-            x = rows[start:end]
-            h = torch.nn.functional.silu(x @ gate[g]) * (x @ up[g])
-            y = (h @ down[g].t()).float() * slots[start:end, None]
-            out[start:end] = y.to(rows.dtype)
-        start = end
-    return out

@@ -122,8 +122,9 @@ def _tpe_table(ctx: dict, tokens_per_expert: torch.Tensor) -> torch.Tensor:
     """The ``[R, E]`` count table the planner reads.  A per-rank ``[E]`` row is
     deposited into the world's gathered table (the reference's planner writes
     its row into its peers' meta chunks, planning.py:577-583) and the table of
-    this rank's meta chunk is returned; the caller has to make sure the other
-    ranks' rows are in (``EmulatedWorld.rendezvous``) before the launch."""
+    this rank's meta chunk is returned after a rendezvous of the rank threads, so that
+    every row is in; without rank threads there is nobody to fill the other rows and the
+    call is refused."""
     R, E = int(ctx["R"]), int(ctx["E"])
     assert tokens_per_expert.dtype == torch.int32 and tokens_per_expert.is_contiguous()
     if tokens_per_expert.dim() == 2:
@@ -135,7 +136,13 @@ def _tpe_table(ctx: dict, tokens_per_expert: torch.Tensor) -> torch.Tensor:
     if R == 1:
         return tokens_per_expert.reshape(1, E)
     world, rank = ctx["world"], int(ctx["rank"])
+    if not world.host_threads:
+        raise NotImplementedError(
+            "launch_planning(tokens_per_expert[E]) of one rank needs the other ranks' counts: pass "
+            f"the gathered tokens_per_expert[R={R}, E={E}], or run every rank on its own host "
+            "thread of an EmulatedWorld(host_threads=True)")
     world.deposit_tokens_per_expert(rank, tokens_per_expert)
+    world.rendezvous(rank)
     return world.tpe_table(rank)
 
 

@@ -108,3 +108,60 @@ def launch_prefetch(local_weights, prefetch_buffers, experts_to_copy, rank, num_
         _lib.current_stream(),
     )
     _lib.check(rc, "mep_prefetch")
+
+
+def launch_prefetch_pull(owner_weights, prefetch_buffers, experts_to_copy, rank, scales=None) -> None:
+    """Pull view of ``launch_prefetch`` (not in the reference, whose ranks push): fill the
+    occupied prefetch slots of ONE rank from every owner's experts in one launch,
+    ``pool[rank, b] = owner_weights[e // epn, e % epn]`` for ``e = experts_to_copy[rank, b] >= 0``.
+
+    ``owner_weights``: three ``[R, epn, H, H']`` tensors holding every rank's local experts
+    (what one GPU emulating the R ranks has at hand; rank-strided like a pool);
+    ``prefetch_buffers`` and ``scales`` (three ``(owner_scales[R, epn, ...], pool)`` pairs) as
+    for ``launch_prefetch``.  Leaves in ``pool[rank]`` exactly what the R owners' pushes
+    leave there (the per-rank check of reference tests/test_prefetch.py:448-464)."""
+    assert len(owner_weights) == 3 and len(prefetch_buffers) == 3, \
+        "prefetch requires three owner weight tensors and three prefetch buffers"
+    dtype = owner_weights[0].dtype
+    assert dtype in _ELEM_TYPES, (
+        f"prefetch: unsupported dtype {dtype}; supported: {sorted(str(d) for d in _ELEM_TYPES)}"
+    )
+    assert owner_weights[0].ndim == 4 and prefetch_buffers[0].ndim == 4
+    R, EPN = (int(x) for x in prefetch_buffers[0].shape[:2])
+    device_index = prefetch_buffers[0].device.index
+    assert device_index is not None, "prefetch buffers must be CUDA tensors"
+    for ow, pb in zip(owner_weights, prefetch_buffers, strict=True):
+        assert ow.ndim == 4 and tuple(ow.shape[:2]) == (R, EPN) and ow[0].is_contiguous(), \
+            f"owner weights must be [R, EPN]=[{R}, {EPN}] leading, contiguous within each rank"
+        _validate_pair(ow[0], pb, EPN, R, dtype, device_index)
+        assert (int(ow.stride(0)) * ow.element_size()) % 16 == 0 and ow.data_ptr() % 16 == 0, \
+            "owner weights must be 16-byte aligned rank by rank"
+    assert experts_to_copy.dtype == torch.int32 and experts_to_copy.is_contiguous(), \
+        "experts_to_copy must be contiguous int32 [R, EPN]"
+    assert tuple(experts_to_copy.shape) == (R, EPN), f"experts_to_copy must be [R, EPN]=[{R}, {EPN}]"
+    assert experts_to_copy.device.index == device_index
+    assert 0 <= int(rank) < R, f"rank must be in [0, {R}), got {rank}"
+    owners, pools = list(owner_weights), list(prefetch_buffers)
+    if scales is not None:
+        assert len(scales) == 3, "prefetch scales must contain three owner/pool pairs"
+        assert dtype == torch.uint8, "weight and re-tiled scale tensors must share uint8 copy dtype"
+        for os_, sp in scales:
+            assert tuple(os_.shape[:2]) == (R, EPN) and os_[0].is_contiguous()
+            assert tuple(sp.shape) == tuple(os_.shape) and sp.dtype == os_.dtype
+            assert os_.device.index == device_index and sp.device.index == device_index
+            assert sp[0].is_contiguous()
+            retile_for_prefetch(os_[0])  # same size rule as the reference
+            owners.append(os_)
+            pools.append(sp)
+    n = len(owners)
+    arr_p = (C.c_void_p * n)
+    arr_i = (C.c_int64 * n)
+    bytes_per = [t[0].nbytes // EPN for t in owners]
+    rc = _lib.lib().mep_prefetch_pull(
+        n, arr_p(*[t.data_ptr() for t in owners]),
+        arr_i(*[int(t.stride(0)) * t.element_size() for t in owners]),
+        arr_p(*[p.data_ptr() for p in pools]),
+        arr_i(*[int(p.stride(0)) * p.element_size() for p in pools]),
+        arr_i(*bytes_per), experts_to_copy.data_ptr(), int(rank), EPN, R, _lib.current_stream(),
+    )
+    _lib.check(rc, "mep_prefetch_pull")

@@ -80,6 +80,8 @@ int main() {
   std::printf("libmoonep_hip v%d: S=%d H=%d K=%d E=%d R=%d tp=%d NvS=%d rank=%d\n", mep_version(), S, H,
               K, E, R, tp, NvS, rank);
   int bad = 0;
+  if (mep_version() != 200) { std::printf("FAIL header and library disagree on the ABI version\n"); return 2; }
+  MEP_OK_(mep_init());   // per-device set-up, outside any capture
 
   // ---- routing of all ranks (skewed: low expert ids are popular), counts table
   std::vector<int32_t> topk((size_t)R * N), tpe((size_t)R * E, 0);

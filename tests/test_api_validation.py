@@ -154,3 +154,50 @@ def test_grouped_gemm_rejects_paddings_that_split_a_tile():
             launch_grouped_gemm_nt(x, x, x, token_padding=tp)
         with pytest.raises(AssertionError, match="multiple of 128"):
             grouped_ffn_hip(x, None, x, x, x, x, token_padding=tp)
+
+
+def test_the_reference_import_name_resolves_to_this_package():
+    """``from moonep import Buffer, MoonEPCommPlan`` (reference moonep/__init__.py:1-9) and the
+    reference's module paths of the launchers work unchanged."""
+    import moonep
+    from moonep import Buffer as B2, MoonEPCommPlan as P2
+    from moonep.combine_prologue import launch_combine_prologue
+    from moonep.dispatch_epilogue import launch_dispatch_epilogue
+    from moonep.planning import launch_planning
+    import moonep.api
+
+    assert B2 is Buffer and P2 is MoonEPCommPlan
+    assert moonep.api is api and moonep.__all__ == ["Buffer", "MoonEPCommPlan"]
+    assert launch_dispatch_epilogue.__module__ == "moonep_amd.dispatch"
+    assert launch_combine_prologue.__module__ == "moonep_amd.combine"
+    assert launch_planning.__module__ == "moonep_amd.planning"
+
+
+def test_per_rank_counts_need_rank_threads():
+    """A one-rank tokens_per_expert[E] reaches the planner only through the gathered table,
+    which nobody fills without rank threads: refused before any device access."""
+    from moonep_amd.planning import _tpe_table
+
+    class World:
+        host_threads = False
+
+    ctx = dict(R=4, E=8, rank=1, world=World())
+    with pytest.raises(NotImplementedError, match=r"tokens_per_expert\[R=4, E=8\]"):
+        _tpe_table(ctx, torch.zeros(8, dtype=torch.int32))
+    table = torch.zeros(4, 8, dtype=torch.int32)
+    assert _tpe_table(ctx, table) is table
+
+
+def test_reduce_grad_phase_argument_and_pool_checks_are_host_side():
+    """Shape / dtype / stride checks of the (local, pool) pairs in own words; the messages the
+    reference's tests match by substring are kept."""
+    local = torch.zeros(2, 4, 4)
+    pool = torch.zeros(3, 2, 4, 4)
+    with pytest.raises(AssertionError, match="unsupported weight dtype"):
+        api._check_local_pool_pairs("prefetch_weight", [local], [pool], 2, 3, dtypes=(torch.bfloat16,))
+    with pytest.raises(AssertionError, match=r"must be \[epn=5"):
+        api._check_local_pool_pairs("reduce_grad", [local], [pool], 5, 3, dtypes=(torch.float32,))
+    with pytest.raises(AssertionError, match=r"pool must be \[R=4, epn=2"):
+        api._check_local_pool_pairs("reduce_grad", [local], [pool], 2, 4, dtypes=(torch.float32,))
+    with pytest.raises(AssertionError, match="3 dimensions"):
+        api._check_local_pool_pairs("reduce_grad", [local[0]], [pool[:, 0]], 4, 3, dtypes=(torch.float32,))

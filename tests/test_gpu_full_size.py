@@ -23,15 +23,15 @@ from moonep_amd.combine import launch_combine
 from moonep_amd.dispatch import launch_dispatch
 from moonep_amd.grad_reduce import launch_grad_reduce
 from moonep_amd.planning import allocate_planning_outputs, launch_planning, launch_planning_all_ranks
-from moonep_amd.prefetch import launch_prefetch
+from moonep_amd.prefetch import launch_prefetch, launch_prefetch_pull
 from oracle import ops_oracle as oo
 from oracle import planner_oracle as po
 
 pytestmark = pytest.mark.gpu
 
 R, K, TP = 8, 8, 128
-SWEEP = [(4096, 7168, 256, mv) for mv in (0.0, 0.5, 2.0, 4.0)] + \
-        [(8192, 4096, 128, mv) for mv in (0.0, 0.5, 1.0, 4.0)] + \
+SWEEP = [(4096, 7168, 256, mv) for mv in (0.0, 0.5, 1.0, 2.0, 4.0)] + \
+        [(8192, 4096, 128, mv) for mv in (0.0, 0.5, 1.0, 2.0, 4.0)] + \
         [(8192, 7168, 384, 1.0)]      # the configuration of the reference's own figure
 
 
@@ -138,7 +138,22 @@ def test_prefetch_and_grad_reduce_at_the_real_shape_with_the_planners_table(cuda
                 else:       # not this owner's: still the sentinel, or an earlier owner's expert
                     assert got[0] == got[1] and (got[0] == SENT or got[0] == e / 8), (owner, d, b, got)
         del local
-    del pool
+    # ---- the pull view: the fullest rank's slots from all owners in one launch
+    pool.fill_(SENT)
+    ids = (torch.arange(R * epn, device=cuda).to(torch.bfloat16) / 8).view(R, epn)
+    all_local = ids[:, :, None, None].expand(R, epn, H, Hp).contiguous()                 # 7.5 GB
+    n_full, fullest = max((int((etc[r] >= 0).sum()), r) for r in range(R))
+    launch_prefetch_pull((all_local,) * 3, (pool,) * 3, etc_dev, rank=fullest)
+    torch.cuda.synchronize()
+    flat = pool.view(R * epn, H * Hp)
+    lo, hi = flat.min(dim=1).values.float().cpu(), flat.max(dim=1).values.float().cpu()
+    for d in range(R):
+        for b in range(epn):
+            e = int(etc[d, b])
+            want = e / 8 if (d == fullest and e >= 0) else SENT
+            assert (float(lo[d * epn + b]), float(hi[d * epn + b])) == (want, want), (d, b, e)
+    print(f"pull: rank {fullest} filled {n_full} slots", flush=True)
+    del pool, all_local
     torch.cuda.empty_cache()
 
     # ---- grad reduce: slot (src, b) = src*64 + b, local grad of expert le = 1000 + le

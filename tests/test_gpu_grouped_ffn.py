@@ -14,12 +14,15 @@ from moonep_amd.ffn import grouped_ffn_hip, launch_grouped_gemm_nt
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["128", "256"])
-def row_tile(request, monkeypatch):
+@pytest.fixture(autouse=True, params=[128, 256])
+def row_tile(request):
     """Every test runs on both row tilings of the grouped kernel (the library picks by shape;
     the small shapes here would only ever see one of them)."""
-    monkeypatch.setenv("MEP_GEMM_ROW_TILE", request.param)
-    return request.param
+    from moonep_amd import _lib
+
+    _lib.check(_lib.lib().mep_set_gemm_row_tile(request.param), "mep_set_gemm_row_tile")
+    yield request.param
+    _lib.check(_lib.lib().mep_set_gemm_row_tile(0), "mep_set_gemm_row_tile")
 
 
 def _groups(G, M, seed, tail):
@@ -105,8 +108,8 @@ def test_no_rows_at_all(cuda):
 
 
 def test_grouped_ffn_matches_the_torch_consumer(cuda):
-    """Same contract as moonep_amd.moe.grouped_ffn (library GEMMs per group)."""
-    from moonep_amd.moe import grouped_ffn
+    """Same contract as the plain-PyTorch consumer (library GEMMs per group)."""
+    from tests.util import grouped_ffn
 
     NvS, H, Hp, G = 1536, 512, 256, 8
     g = torch.Generator().manual_seed(11)

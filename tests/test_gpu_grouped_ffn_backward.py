@@ -16,12 +16,15 @@ from moonep_amd import ffn
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["128", "256"])
-def row_tile(request, monkeypatch):
+@pytest.fixture(autouse=True, params=[128, 256])
+def row_tile(request):
     """Every test runs on both row tilings of the grouped kernel (the library picks by shape;
     the small shapes here would only ever see one of them)."""
-    monkeypatch.setenv("MEP_GEMM_ROW_TILE", request.param)
-    return request.param
+    from moonep_amd import _lib
+
+    _lib.check(_lib.lib().mep_set_gemm_row_tile(request.param), "mep_set_gemm_row_tile")
+    yield request.param
+    _lib.check(_lib.lib().mep_set_gemm_row_tile(0), "mep_set_gemm_row_tile")
 
 
 def _groups(G, M, seed, tail):

@@ -10,6 +10,7 @@ import pytest
 import torch
 
 from moonep_amd import moe, routing
+from tests.util import grouped_ffn
 
 pytestmark = pytest.mark.gpu
 
@@ -47,7 +48,7 @@ def test_moe_layer_forward_backward_matches_dense(cuda, sigma):
     if sigma > 0:
         assert bool((etc >= 0).any()), "the skewed routing must exercise prefetch slots"
     views = [moe.group_compute_views(group, etc, m) for m in master]
-    y = torch.stack([moe.grouped_ffn(rows[r], slots[r], cu[r], views[0][r], views[1][r], views[2][r])
+    y = torch.stack([grouped_ffn(rows[r], slots[r], cu[r], views[0][r], views[1][r], views[2][r])
                      for r in range(R)])
     out = moe.group_combine(group, plans, y)
     (out.float() * gout).sum().backward()

@@ -12,7 +12,8 @@ import pytest
 import torch
 
 from moonep_amd.grad_reduce import launch_grad_reduce
-from moonep_amd.prefetch import launch_prefetch, prefetch_retile_nbytes, retile_for_prefetch
+from moonep_amd.prefetch import (launch_prefetch, launch_prefetch_pull, prefetch_retile_nbytes,
+                                 retile_for_prefetch)
 from oracle import ops_oracle as oo
 
 pytestmark = pytest.mark.gpu
@@ -197,6 +198,82 @@ def test_prefetch_with_scales_and_large_offsets(cuda):
     torch.cuda.synchronize()
     assert torch.equal(pool[2, 1], local[1])
     assert not bool(pool[2, 0].any()) and not bool(pool[:2].any())
+
+
+PULL_CASES = ["rect_tiles", "random_holes_dups", "fan_in", "empty", "uint8_packed", "offset_128B_pool"]
+
+
+@pytest.mark.parametrize("case", [c for c in PREFETCH_CASES if c[0] in PULL_CASES],
+                         ids=[c[0] for c in PREFETCH_CASES if c[0] in PULL_CASES])
+def test_prefetch_pull_fills_one_ranks_slots_like_all_owner_pushes(cuda, case):
+    """The pull view (one launch per destination rank, reading every owner's experts) leaves in
+    pool[rank] what the R owner pushes leave there, and touches nothing else: slots of other
+    ranks, free slots and the padding between ranks keep their sentinel (the per-rank check of
+    reference tests/test_prefetch.py:448-464)."""
+    name, R, epn, H, Hp, dtype, plan_name, seed, pad = case
+    print(f"prefetch pull case {name}", flush=True)
+    etc = PLANS[plan_name](R, epn, seed)
+    sent = SENTINEL if dtype.is_floating_point else (0xAB if dtype == torch.uint8 else 123)
+    g = torch.Generator().manual_seed(300 + seed)
+    shapes = [(H, Hp), (H, Hp), (Hp, H)]
+    owners_ref, owners_dev, ref_pools = [], [], []
+    for t, shp in enumerate(shapes):
+        # every owner's local experts side by side, with padding between the owners too
+        _, ow = strided_pool(R, (epn, *shp), dtype, 16 * (t + 1), 0, "cpu")
+        ow.copy_(_fill((R, epn, *shp), dtype, g))
+        _, od = strided_pool(R, (epn, *shp), dtype, 16 * (t + 1), 0, cuda)
+        od.copy_(ow)
+        owners_ref.append(ow)
+        owners_dev.append(od)
+        _, rp = strided_pool(R, (epn, *shp), dtype, pad * (t + 1), sent, "cpu")
+        for owner in range(R):
+            oo.prefetch(ow[owner], rp, etc, owner)
+        ref_pools.append(rp)
+    etc_dev = etc.to(cuda)
+    for rank in range(R):
+        dev_pools, dev_backing = [], []
+        for t, shp in enumerate(shapes):
+            lead = 64 * (t + 1) if name.startswith("offset") else 0
+            bk, dp = strided_pool(R, (epn, *shp), dtype, pad * (t + 1), sent, cuda, lead)
+            dev_pools.append(dp)
+            dev_backing.append(bk)
+        launch_prefetch_pull(tuple(owners_dev), tuple(dev_pools), etc_dev, rank=rank)
+        torch.cuda.synchronize()
+        for t in range(3):
+            got = dev_pools[t].cpu()
+            assert torch.equal(got[rank], ref_pools[t][rank]), f"rank {rank} tensor {t}"
+            others = [d for d in range(R) if d != rank]
+            assert (got[others] == sent).all(), "a pull wrote into another rank's slots"
+            stride, numel = dev_pools[t].stride(0), dev_pools[t][0].numel()
+            if stride > numel:
+                assert (dev_backing[t].cpu().view(R, stride)[:, numel:] == sent).all()
+
+
+def test_prefetch_pull_with_scales(cuda):
+    R, epn, H, Hp = 4, 3, 256, 256
+    etc = torch.full((R, epn), -1, dtype=torch.int32)
+    for d in range(R):
+        etc[d, 0] = ((d + 1) % R) * epn + 2
+        etc[d, 2] = ((d + 3) % R) * epn + 1
+    g = torch.Generator().manual_seed(6)
+    scale_shape = (64, 64)
+    own_w = [_fill((R, epn, H, Hp), torch.uint8, g) for _ in range(3)]
+    own_s = [torch.randn((R, epn, *scale_shape), generator=g) for _ in range(3)]
+    ref_w = [torch.full((R, epn, H, Hp), 0xAB, dtype=torch.uint8) for _ in range(3)]
+    ref_s = [torch.full((R, epn, *scale_shape), SENTINEL) for _ in range(3)]
+    dev_w = [x.to(cuda) for x in ref_w]
+    dev_s = [x.to(cuda) for x in ref_s]
+    dow, dos = [x.to(cuda) for x in own_w], [x.to(cuda) for x in own_s]
+    for rank in range(R):
+        for t in range(3):
+            oo.prefetch(own_w[t][rank], ref_w[t], etc, rank)
+            oo.prefetch(own_s[t][rank], ref_s[t], etc, rank)
+        launch_prefetch_pull(tuple(dow), tuple(dev_w), etc.to(cuda), rank=rank,
+                             scales=tuple((dos[t], dev_s[t]) for t in range(3)))
+    torch.cuda.synchronize()
+    for t in range(3):
+        assert torch.equal(dev_w[t].cpu(), ref_w[t])
+        assert torch.equal(dev_s[t].cpu().view(torch.int32), ref_s[t].view(torch.int32))
 
 
 # ---------------------------------------------------------------- grad reduce

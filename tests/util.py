@@ -49,3 +49,24 @@ def traceable_weights(S: int, K: int, rank: int) -> torch.Tensor:
     """fp32 whose bit pattern is a ramp: exact round trips are visible."""
     ramp = torch.arange(S * K, dtype=torch.int32) + rank * S * K + 1
     return ramp.view(torch.float32).reshape(S, K)
+
+
+def grouped_ffn(rows, slots, cu_seqlens, gate, up, down):
+    """Plain-PyTorch consumer of one rank's dispatched rows (library GEMMs per group, group
+    bounds read on the host): what the HIP expert FFN is checked against.
+
+    rows [NvS,H] bf16, slots [NvS] fp32 route weights, cu_seqlens [2*epn]
+    (padded end offset of every group), gate/up/down [2*epn,H,H'] compute
+    views.  Group g applies ``w * (silu(x @ gate[g]) * (x @ up[g])) @ down[g].T``
+    to its rows; rows outside every group are zero (reference README.md:43-58).
+    """
+    out = torch.zeros_like(rows)
+    start = 0
+    for g, end in enumerate(cu_seqlens.tolist()):
+        if end > start:
+            x = rows[start:end]
+            h = torch.nn.functional.silu(x @ gate[g]) * (x @ up[g])
+            y = (h @ down[g].t()).float() * slots[start:end, None]
+            out[start:end] = y.to(rows.dtype)
+        start = end
+    return out
