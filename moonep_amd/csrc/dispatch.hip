@@ -331,13 +331,19 @@ extern "C" int mep_dispatch(const void* hidden_SH, const float* w_SK, const int3
   a.zblocks = zblocks;
   dim3 grid(a.tok_blocks + zblocks);
   hipStream_t st = (hipStream_t)stream;
+  // rows that are a whole number of 1-KiB wave tiles (H % 512 == 0, up to H = 8192) pass
+  // through registers in one go; any other H % 8 == 0 takes the strided loop
   const int nvec = H / 8;
-  if (nvec % 64 == 0 && nvec / 64 == 14) {
-    hipLaunchKernelGGL(dispatch_kernel<14>, grid, dim3(kBlock), 0, st, a);
-  } else if (nvec % 64 == 0 && nvec / 64 == 8) {
-    hipLaunchKernelGGL(dispatch_kernel<8>, grid, dim3(kBlock), 0, st, a);
-  } else {
-    hipLaunchKernelGGL(dispatch_kernel<0>, grid, dim3(kBlock), 0, st, a);
+  const int tiles = nvec % 64 == 0 ? nvec / 64 : 0;
+  switch (tiles) {
+#define MEP_DISPATCH_CASE(NV) \
+    case NV: hipLaunchKernelGGL(dispatch_kernel<NV>, grid, dim3(kBlock), 0, st, a); break;
+    MEP_DISPATCH_CASE(1) MEP_DISPATCH_CASE(2) MEP_DISPATCH_CASE(3) MEP_DISPATCH_CASE(4)
+    MEP_DISPATCH_CASE(5) MEP_DISPATCH_CASE(6) MEP_DISPATCH_CASE(7) MEP_DISPATCH_CASE(8)
+    MEP_DISPATCH_CASE(9) MEP_DISPATCH_CASE(10) MEP_DISPATCH_CASE(11) MEP_DISPATCH_CASE(12)
+    MEP_DISPATCH_CASE(13) MEP_DISPATCH_CASE(14) MEP_DISPATCH_CASE(15) MEP_DISPATCH_CASE(16)
+#undef MEP_DISPATCH_CASE
+    default: hipLaunchKernelGGL(dispatch_kernel<0>, grid, dim3(kBlock), 0, st, a); break;
   }
   return mep_launch_status();
 }

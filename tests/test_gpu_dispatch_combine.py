@@ -54,6 +54,11 @@ CASES = [
     ("h7168_rows", 64, 7168, 8, 4, 8, 32, ("biased", 1.0)),
     ("h4096_rows", 48, 4096, 8, 2, 8, 16, ("biased", 2.0)),
     ("k32", 8, 1024, 32, 8, 4, 8, ("biased", 1.0)),
+    # rows of 3, 10 and 16 whole 1-KiB wave tiles, and one just past a tile (the strided loop)
+    ("h1536_rows", 40, 1536, 4, 2, 4, 8, ("biased", 1.0)),
+    ("h5120_rows", 24, 5120, 6, 4, 4, 16, ("biased", 1.5)),
+    ("h8192_rows", 24, 8192, 8, 2, 8, 16, ("biased", 1.0)),
+    ("h8200_rows", 12, 8200, 2, 2, 4, 4, ("biased", 1.0)),
 ]
 
 
