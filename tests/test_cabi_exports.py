@@ -122,6 +122,41 @@ def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
     assert lib.mep_swiglu_bwd(A, A, None, None, A, 4, A, A, A, None, 128, 128, None) == -1
 
 
+def test_argument_checks_of_the_entry_points_added_with_abi_200():
+    import ctypes as C
+
+    lib = _lib.lib()
+    A = 0x10000
+    assert lib.mep_version() == _lib.ABI_VERSION == 200
+    # pull prefetch: host arrays of pointers / strides / sizes
+    arr_p, arr_i = (C.c_void_p * 3), (C.c_int64 * 3)
+    ok = dict(owners=arr_p(A, A, A), ostride=arr_i(4096, 4096, 4096), pool=arr_p(A, A, A),
+              pstride=arr_i(4096, 4096, 4096), per=arr_i(1024, 1024, 1024))
+
+    def pull(n=3, rank=0, epn=4, R=2, etc=A, **kw):
+        a = dict(ok, **kw)
+        return lib.mep_prefetch_pull(n, a["owners"], a["ostride"], a["pool"], a["pstride"], a["per"], etc,
+                                     rank, epn, R, None)
+
+    assert pull(etc=None) == -1
+    assert pull(n=7) == -1                                   # more than six tensors
+    assert pull(rank=2) == -1                                # rank outside [0, R)
+    assert pull(per=arr_i(1024, 1000, 1024)) == -2           # bytes per expert not a multiple of 16
+    assert pull(ostride=arr_i(4096, 2048, 4096)) == -1       # owners' experts would overlap
+    assert pull(pool=arr_p(A, A + 8, A)) == -4               # misaligned pool
+    assert pull(owners=arr_p(A, None, A)) == -1
+    # duplicate kernels: the CU bound is an ordinary int; the usual checks come first
+    assert lib.mep_dispatch_epilogue(None, A, A, A, 64, 64, 32, None) == -1
+    assert lib.mep_combine_prologue(A, A, A, A, 64, 60, 0, None) == -2        # H % 8 != 0
+    assert lib.mep_combine_prologue(A + 2, A, A, A, 64, 64, 1, None) == -4
+    # the GEMM tiling hook takes 0, 128 or 256
+    assert lib.mep_set_gemm_row_tile(7) == -1 and lib.mep_set_gemm_row_tile(256) == 0
+    assert lib.mep_set_gemm_row_tile(0) == 0
+    # the dst encoding bound is checked by every consumer of dst, not only by the planner
+    assert lib.mep_dispatch(A, None, A, A, A, 1 << 30, None, 0, 0, 4, 64, 2, 2, 4, 1 << 30, 8, 0, None) == -2
+    assert lib.mep_combine(A, 1 << 30, None, 0, A, A, None, 4, 64, 2, 2, 1 << 30, 0, None) == -2
+
+
 def test_static_scratch_entry_point_rejects_inputs_beyond_its_fixed_size():
     """mep_build_dedup_static allocates nothing: its scratch is a fixed 1 MiB device
     array; a larger input is refused with its own error code before any device call."""
