@@ -689,7 +689,8 @@ class Buffer:
         epn = int(ctx["E"]) // R
         local_weights = (local_gate_weight, local_up_weight, local_down_weight)
         pools = (gate_prefetch_buffer, up_prefetch_buffer, down_prefetch_buffer)
-        assert None not in (*local_weights, *pools), "prefetch_weight tensors must be provided together"
+        assert all(t is not None for t in (*local_weights, *pools)), \
+            "prefetch_weight tensors must be provided together"
         _check_local_pool_pairs("prefetch_weight", local_weights, pools, epn, R, dtypes=_ELEM_TYPES)
         local_scales = (local_gate_scale, local_up_scale, local_down_scale)
         scale_pools = (gate_scale_prefetch_buffer, up_scale_prefetch_buffer,
@@ -775,7 +776,8 @@ class Buffer:
         epn = int(ctx["E"]) // R
         local_grads = (local_gate_grad, local_up_grad, local_down_grad)
         pools = (gate_reduce_buffer, up_reduce_buffer, down_reduce_buffer)
-        assert None not in (*local_grads, *pools), "reduce_grad tensors must be provided together"
+        assert all(t is not None for t in (*local_grads, *pools)), \
+            "reduce_grad tensors must be provided together"
         assert isinstance(plan, MoonEPCommPlan), "Buffer.reduce_grad: plan is required"
         assert phase in ("both", "reduce", "clear"), f"phase must be both, reduce or clear, got {phase!r}"
         _check_local_pool_pairs("reduce_grad", local_grads, pools, epn, R, dtypes=(torch.float32,))
