@@ -44,13 +44,16 @@ struct PlanLds {
   static constexpr int FIXED = 2 * NT;
 };
 
-template <int NT, bool kLdsTables>
+// RC, KC: the number of ranks and top-k as compile-time constants (0: taken
+// from the arguments); the planner is a chain of dependent instructions, and
+// a kernel that knows them drops the loops, clamps and alternative paths
+template <int NT, bool kLdsTables, int RC = 0, int KC = 0>
 __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   using L = PlanLds<NT>;
   constexpr int NW = L::NW;
   constexpr int W4 = L::W4;
   extern __shared__ int smem[];
-  const int E = a.E, R = a.R, epn = a.epn, tp = a.tp, NvS = a.NvS, K = a.K;
+  const int E = a.E, R = RC > 0 ? RC : a.R, epn = a.epn, tp = a.tp, NvS = a.NvS, K = KC > 0 ? KC : a.K;
   const int N = a.S * K;
   const int CAP = N;
   int* s_cnt = smem;             // [E] tokens per expert, all ranks
@@ -98,21 +101,92 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   }
   const int rank = a.rank0 + blockIdx.y;
   const bool writer = blockIdx.x == 0;  // one workgroup per rank stores the small outputs
+  const int* topk = a.topk + (size_t)blockIdx.y * N;
+  const int t0 = blockIdx.x * a.tok_per_wg;
+  const int t1 = min(t0 + a.tok_per_wg, a.S);
+  const int e0 = t0 * K;
+  const int n = (t1 - t0) * K;  // <= NT
 
-  // ---- counts per expert, per home group --------------------------------
+  // ---- every load whose address is known now goes out before anything waits ----
+  // (the planner is a chain of latencies; beside a stream of other traffic a
+  // load issued late costs two to three times as much)
+  int e = -1;  // expert of my entry
+  if (tid < n) e = topk[e0 + tid];
+  int tv[8];   // counts of expert `tid` on the first eight ranks (clamped row: no branch)
+  if (tid < E) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) tv[j] = a.tpe[(j < R ? j : R - 1) * E + tid];
+  }
+  // Per expert, this rank's entries that precede the workgroup's slice: needs
+  // nothing from the plan and is only used when the entries are resolved, so it
+  // runs beside the planning phases.  Wave 0 plans alone in the first of them
+  // (the serial greedy) while every other wave counts; in the two phases that
+  // follow, waves 1..R plan (one per rank) and the waves above them count.  Each
+  // part's first loads are issued one phase ahead.  With more ranks than that
+  // leaves counting waves for, the first phase takes all of it.
+  constexpr int HWB = NW / 2 + 1;       // first wave that counts in the later phases
+  constexpr int NA = NT - 64, NB = NT - HWB * 64;
+  const int ta = tid - 64, tb = tid - HWB * 64;
+  const bool count_a = wave >= 1, count_b = wave >= HWB;
+  const bool hist_vec = (((uintptr_t)topk) & 15) == 0;
+  const bool spread = R < HWB;
+  const int nv = hist_vec ? e0 >> 2 : 0;  // 16-byte vectors
+  const int hb1 = spread ? (int)(((int64_t)nv * 15) >> 5) : nv;
+  const int hb2 = spread ? (int)(((int64_t)nv * 24) >> 5) : nv;
+  const int4* t4 = (const int4*)topk;
+  // loads v[u] = vector (b + t + u*nt) for those below `end`
+  auto hist_load = [&](auto& v, int b, int end, int t, int nt) {
+    constexpr int G = sizeof(v) / sizeof(v[0]);
+#pragma unroll
+    for (int u = 0; u < G; ++u)
+      if (b + t + u * nt < end) v[u] = t4[b + t + u * nt];
+  };
+  // an id outside [0, E) counts into a word nobody reads: no branch per atomic
+  auto bin = [&](int x) { return (unsigned)x < (unsigned)E ? s_hist + x : s_bal; };
+  auto hist_count = [&](const auto& v, int b, int end, int t, int nt) {
+    constexpr int G = sizeof(v) / sizeof(v[0]);
+#pragma unroll
+    for (int u = 0; u < G; ++u)
+      if (b + t + u * nt < end) {
+        atomicAdd(bin(v[u].x), 1);
+        atomicAdd(bin(v[u].y), 1);
+        atomicAdd(bin(v[u].z), 1);
+        atomicAdd(bin(v[u].w), 1);
+      }
+  };
+  // counts [b, end) given its first group already loaded into v
+  auto hist_part = [&](auto& v, int b, int end, int t, int nt) {
+    constexpr int G = sizeof(v) / sizeof(v[0]);
+    hist_count(v, b, end, t, nt);
+    for (int i = b + G * nt; i < end; i += G * nt) {
+      hist_load(v, i, end, t, nt);
+      hist_count(v, i, end, t, nt);
+    }
+  };
+  int4 ha[4], hb[6], hc[6];
+  if (count_a) hist_load(ha, 0, hb1, ta, NA);
+
   for (int i = tid; i < R; i += NT) {
     s_gt[i] = 0; s_from[i] = -1; s_quota[i] = 0; s_stat1[i] = 0; s_nrem[i] = 0;
   }
   for (int i = tid; i < W4 * E; i += NT) s_wcnt[i] = 0;
   for (int i = tid; i < E; i += NT) s_hist[i] = 0;
   __syncthreads();
-  for (int e = tid; e < E; e += NT) {
+
+  // ---- counts per expert, per home group --------------------------------
+  const int epn_shift = (epn & (epn - 1)) == 0 ? 31 - __clz(epn) : -1;
+  for (int ee = tid; ee < E; ee += NT) {
     int c = 0, p = 0;
     for (int r0 = 0; r0 < R; r0 += 8) {  // eight independent loads in flight
       int v[8];
+      if (ee == tid && r0 == 0) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j)  // clamped row: no branch between the loads
-        v[j] = a.tpe[(r0 + j < R ? r0 + j : R - 1) * E + e];
+        for (int j = 0; j < 8; ++j) v[j] = tv[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          v[j] = a.tpe[(r0 + j < R ? r0 + j : R - 1) * E + ee];
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int x = r0 + j < R ? v[j] : 0;
@@ -120,83 +194,100 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
         c += x;
       }
     }
-    s_cnt[e] = c; s_prev[e] = p; s_rem[e] = c;
-    const int home = e / epn;
-    for (int d = 0; d < R; ++d) alloc[e * R + d] = (d == home) ? c : 0;
+    s_cnt[ee] = c; s_prev[ee] = p; s_rem[ee] = c;
+    const int home = epn_shift >= 0 ? ee >> epn_shift : ee / epn;
+    for (int d = 0; d < R; ++d) alloc[ee * R + d] = (d == home) ? c : 0;
     atomicAdd(&s_gt[home], c);
   }
   __syncthreads();
 
-  // ---- receivers and quotas (wave 0) | histogram of earlier entries -------
+  // ---- receivers and quotas (wave 0) | my entry among those of my wave | histogram
   // Each receiver is filled exactly once (to capacity), so z[h][u] of the
   // reference (tests/planning_reference.py:85-96) is stored per receiver.
-  // The upper three quarters of the waves meanwhile count, per expert, this rank's
-  // entries that precede the workgroup's slice: that needs nothing from the
-  // plan and hides behind the serial greedy loops.
-  const int* topk = a.topk + (size_t)blockIdx.y * N;
-  const int t0 = blockIdx.x * a.tok_per_wg;
-  const int t1 = min(t0 + a.tok_per_wg, a.S);
-  const int e0 = t0 * K;
-  const int n = (t1 - t0) * K;  // <= NT
   // (value, index) pairs travel through one reduction as value*128 + index
   // code whenever the counts leave 7 bits of room
   const bool packed_key = (int64_t)R * CAP < (1 << 24);
   if (wave == 0) {
-    // lane r keeps the balance of rank r (and of rank r + 64)
-    int b0 = lane < R ? s_gt[lane] - CAP : 0;
-    int b1 = lane + 64 < R ? s_gt[lane + 64] - CAP : 0;
-    const bool v0 = lane < R, v1 = lane + 64 < R;
-    for (int it = 0; it < R; ++it) {
-      int hv, h, uv, u;
-      if (packed_key) {
+    if (packed_key && R <= 16) {
+      // One DPP row holds every rank: lane r keeps the balance of rank r and what
+      // rank r receives.  No branch inside an iteration; the two reductions are
+      // independent and interleave.
+      const bool v0 = lane < R;
+      int b0 = v0 ? s_gt[lane] - CAP : 0;
+      int from = -1, quota = 0;
+      for (int it = 0; it < R; ++it) {
         int kx = v0 ? b0 * 128 + (127 - lane) : INT32_MIN;  // max: first index wins ties
         int kn = v0 ? b0 * 128 + lane : INT32_MAX;          // min: first index wins ties
-        if (v1) { kx = mep_imax(kx, b1 * 128 + (63 - lane)); kn = mep_imin(kn, b1 * 128 + lane + 64); }
-        kx = R <= 16 ? mep_row_max(kx) : mep_wave_max(kx);
-        kn = R <= 16 ? mep_row_min(kn) : mep_wave_min(kn);
-        hv = kx >> 7; h = 127 - (kx & 127);
-        uv = kn >> 7; u = kn & 127;
-      } else {
-        int mx = v0 ? b0 : INT32_MIN, mxi = lane;
-        if (v1 && b1 > mx) { mx = b1; mxi = lane + 64; }
-        int mn = v0 ? b0 : INT32_MAX, mni = lane;
-        if (v1 && b1 < mn) { mn = b1; mni = lane + 64; }
-        mep_wave_argmax_first(mx, mxi, hv, h);
-        mep_wave_argmin_first(mn, mni, uv, u);
+        kx = mep_row_max(kx);
+        kn = mep_row_min(kn);
+        const int hv2 = kx >> 7, h = 127 - (kx & 127);
+        const int uv = kn >> 7, u = kn & 127;
+        if (hv2 <= 0 || uv >= 0) break;
+        const int move = -uv;
+        b0 = lane == h ? b0 - move : b0;
+        const bool recv = lane == u;
+        b0 = recv ? 0 : b0;
+        from = recv ? h : from;
+        quota = recv ? move : quota;
       }
-      if (hv <= 0 || uv >= 0) break;
-      const int move = -uv;
-      if (lane == (h & 63)) { if (h < 64) b0 -= move; else b1 -= move; }
-      if (lane == (u & 63)) { if (u < 64) b0 = 0; else b1 = 0; }
-      if (lane == 0) { s_from[u] = h; s_quota[u] = move; }
-    }
-  } else if (wave >= NW / 4) {
-    constexpr int HT = NT - (NW / 4) * 64;  // threads counting
-    const int ht = tid - (NW / 4) * 64;
-    int done = 0;
-    if ((((uintptr_t)topk) & 15) == 0) {  // 16-byte loads, four in flight
-      const int nv = e0 >> 2;
-      const int4* t4 = (const int4*)topk;
-      for (int i = ht; i < nv; i += 4 * HT) {
-        int4 v[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (i + u * HT < nv) v[u] = t4[i + u * HT];
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (i + u * HT < nv) {
-            if ((unsigned)v[u].x < (unsigned)E) atomicAdd(&s_hist[v[u].x], 1);
-            if ((unsigned)v[u].y < (unsigned)E) atomicAdd(&s_hist[v[u].y], 1);
-            if ((unsigned)v[u].z < (unsigned)E) atomicAdd(&s_hist[v[u].z], 1);
-            if ((unsigned)v[u].w < (unsigned)E) atomicAdd(&s_hist[v[u].w], 1);
-          }
+      if (v0) { s_from[lane] = from; s_quota[lane] = quota; }
+    } else {
+      // lane r keeps the balance of rank r (and of rank r + 64)
+      int b0 = lane < R ? s_gt[lane] - CAP : 0;
+      int b1 = lane + 64 < R ? s_gt[lane + 64] - CAP : 0;
+      const bool v0 = lane < R, v1 = lane + 64 < R;
+      for (int it = 0; it < R; ++it) {
+        int hv2, h, uv, u;
+        if (packed_key) {
+          int kx = v0 ? b0 * 128 + (127 - lane) : INT32_MIN;
+          int kn = v0 ? b0 * 128 + lane : INT32_MAX;
+          if (v1) { kx = mep_imax(kx, b1 * 128 + (63 - lane)); kn = mep_imin(kn, b1 * 128 + lane + 64); }
+          kx = mep_wave_max(kx);
+          kn = mep_wave_min(kn);
+          hv2 = kx >> 7; h = 127 - (kx & 127);
+          uv = kn >> 7; u = kn & 127;
+        } else {
+          int mx = v0 ? b0 : INT32_MIN, mxi = lane;
+          if (v1 && b1 > mx) { mx = b1; mxi = lane + 64; }
+          int mn = v0 ? b0 : INT32_MAX, mni = lane;
+          if (v1 && b1 < mn) { mn = b1; mni = lane + 64; }
+          mep_wave_argmax_first(mx, mxi, hv2, h);
+          mep_wave_argmin_first(mn, mni, uv, u);
+        }
+        if (hv2 <= 0 || uv >= 0) break;
+        const int move = -uv;
+        if (lane == (h & 63)) { if (h < 64) b0 -= move; else b1 -= move; }
+        if (lane == (u & 63)) { if (u < 64) b0 = 0; else b1 = 0; }
+        if (lane == 0) { s_from[u] = h; s_quota[u] = move; }
       }
-      done = nv << 2;
     }
-    for (int i = done + ht; i < e0; i += HT) {
-      const int ee = topk[i];
-      if ((unsigned)ee < (unsigned)E) atomicAdd(&s_hist[ee], 1);
+  }
+  // the first loads of the next part of the histogram, before this one's atomics
+  if (count_b && spread) hist_load(hb, hb1, hb2, tb, NB);
+  // Lanes of my wave before me holding the same expert (one ballot per key bit);
+  // the first of them adds the wave's count to the expert's per-wave byte.  Wave 0
+  // does this in the next phase, where it has nothing else to do.
+  if ((unsigned)e >= (unsigned)E) e = -1;  // invalid id: becomes an entry that nobody copies
+  int pos = 0;
+  auto rank_in_wave = [&]() {
+    uint64_t same = __ballot(e >= 0);
+    const int nbits = 32 - __clz(E - 1 > 0 ? E - 1 : 1);
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = (e >> b) & 1;
+      const uint64_t bb = __ballot(bit);
+      same &= bit ? bb : ~bb;
     }
+    if (e >= 0) {
+      pos = __popcll(same & mep_lanes_lt());
+      if (pos == 0)
+        atomicAdd(&s_wcnt[e * W4 + (wave >> 2)], __popcll(same) << (8 * (wave & 3)));
+    }
+  };
+  if (count_a) {
+    rank_in_wave();
+    hist_part(ha, 0, hb1, ta, NA);
+    for (int i = (nv << 2) + ta; i < e0; i += NA)  // what 16-byte loads do not reach
+      atomicAdd(bin(topk[i]), 1);
   }
   __syncthreads();
 
@@ -204,28 +295,52 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   // An (expert, receiver) pair is touched at most once (every step exhausts
   // the expert or the receiver), so alloc[e][d] is a plain store and what
   // stays home is written once at the end.
-  for (int h = wave; h < R; h += NW) {
+  // (waves 1..R, so that wave 0 is free)
+  if (wave == 0) rank_in_wave();
+  if (count_b && spread) {
+    hist_load(hc, hb2, nv, tb, NB);
+    hist_part(hb, hb1, hb2, tb, NB);
+  }
+  for (int h = (wave + NW - 1) % NW; h < R; h += NW) {
     const int es = h * epn;
     if (packed_key && R <= 64 && epn <= 64) {
       // lane r keeps the open quota of receiver r, lane le what is left of
       // the home's expert le
       int q = (lane < R && s_from[lane] == h) ? s_quota[lane] : 0;
       int rem = lane < epn ? s_rem[es + lane] : -1;
-      for (int it = 0; it < R + epn; ++it) {
-        int kq = q > 0 ? q * 128 + (127 - lane) : INT32_MIN;
-        kq = R <= 16 ? mep_row_max(kq) : mep_wave_max(kq);
-        if (kq < 0) break;  // no open quota
-        const int quota = kq >> 7, d = 127 - (kq & 127);
-        int kr = rem >= 0 ? rem * 64 + (63 - lane) : INT32_MIN;
-        kr = epn <= 16 ? mep_row_max(kr) : mep_wave_max(kr);
-        const int best = kr >> 6, le = 63 - (kr & 63);
-        if (best <= 0) break;
-        const int take = best < quota ? best : quota;
-        if (lane == le) {
-          rem -= take;
-          alloc[(es + le) * R + d] = take;
+      if (R <= 16) {  // the receivers fit one DPP row; the two reductions interleave
+        for (int it = 0; it < R + epn; ++it) {
+          int kq = q > 0 ? q * 128 + (127 - lane) : INT32_MIN;
+          int kr = rem >= 0 ? rem * 64 + (63 - lane) : INT32_MIN;
+          kq = mep_row_max(kq);
+          kr = mep_wave_max(kr);
+          const int best = kr >> 6, le = 63 - (kr & 63);
+          if (kq < 0 || best <= 0) break;  // no open quota, or nothing left to move
+          const int quota = kq >> 7, d = 127 - (kq & 127);
+          const int take = best < quota ? best : quota;
+          if (lane == le) {
+            rem -= take;
+            alloc[(es + le) * R + d] = take;
+          }
+          q = lane == d ? q - take : q;
         }
-        if (lane == d) q -= take;
+      } else {
+        for (int it = 0; it < R + epn; ++it) {
+          int kq = q > 0 ? q * 128 + (127 - lane) : INT32_MIN;
+          kq = mep_wave_max(kq);
+          if (kq < 0) break;  // no open quota
+          const int quota = kq >> 7, d = 127 - (kq & 127);
+          int kr = rem >= 0 ? rem * 64 + (63 - lane) : INT32_MIN;
+          kr = mep_wave_max(kr);
+          const int best = kr >> 6, le = 63 - (kr & 63);
+          if (best <= 0) break;
+          const int take = best < quota ? best : quota;
+          if (lane == le) {
+            rem -= take;
+            alloc[(es + le) * R + d] = take;
+          }
+          if (lane == d) q -= take;
+        }
       }
       if (lane < epn) alloc[(es + lane) * R + h] = rem;
       continue;
@@ -249,10 +364,10 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       if (rem <= 0) break;
       const int take = rem < quota ? rem : quota;
       if (lane == 0) {
-        const int e = es + le;
-        alloc[e * R + d] = take;
-        alloc[e * R + h] = rem - take;
-        s_rem[e] = rem - take;
+        const int ex = es + le;
+        alloc[ex * R + d] = take;
+        alloc[ex * R + h] = rem - take;
+        s_rem[ex] = rem - take;
         s_quota[d] = quota - take;
       }
       mep_wave_sync();
@@ -261,25 +376,36 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   __syncthreads();
 
   // ---- layout of every destination: one wave per destination -------------
+  if (count_b && spread) hist_part(hc, hb2, nv, tb, NB);
   const bool tp_pow2 = (tp & (tp - 1)) == 0;
-  const int epn_shift = (epn & (epn - 1)) == 0 ? 31 - __clz(epn) : -1;
-  for (int d = wave; d < R; d += NW) {
+  for (int d = (wave + NW - 1) % NW; d < R; d += NW) {
     const int lo = d * epn, hi = lo + epn;
     int nremote = 0;
-    for (int c = 0; c < E; c += 64) {
-      const int e = c + lane;
-      const bool sel = e < E && (e < lo || e >= hi) && alloc[e * R + d] > 0;
-      const uint64_t m = __ballot(sel);
-      if (sel) {
-        const int slot = nremote + __popcll(m & mep_lanes_lt());
-        if (slot < epn) s_etc[lo + slot] = e;
-        atomicAdd(&s_stat1[epn_shift >= 0 ? e >> epn_shift : e / epn], 1);
+    for (int c0 = 0; c0 < E; c0 += 256) {
+      int av[4];  // four reads in flight
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int ex = c0 + u * 64 + lane;
+        av[u] = ex < E ? alloc[ex * R + d] : 0;
       }
-      nremote += __popcll(m);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int ex = c0 + u * 64 + lane;
+        const bool sel = ex < E && (ex < lo || ex >= hi) && av[u] > 0;
+        const uint64_t m = __ballot(sel);
+        if (sel) {
+          const int slot = nremote + __popcll(m & mep_lanes_lt());
+          if (slot < epn) s_etc[lo + slot] = ex;
+          atomicAdd(&s_stat1[epn_shift >= 0 ? ex >> epn_shift : ex / epn], 1);
+        }
+        nremote += __popcll(m);
+      }
     }
     for (int b = nremote + lane; b < epn; b += 64) s_etc[lo + b] = -1;
     if (lane == 0) s_nrem[d] = nremote;
     mep_wave_sync();
+    if (writer && blockIdx.y == 0)
+      for (int b = lane; b < epn; b += 64) a.etc[lo + b] = s_etc[lo + b];
     const bool mine = writer && d == rank;
     int* cu = a.cu_seqlens + (size_t)blockIdx.y * 2 * epn;
     int* zf = a.zero_fill + (size_t)blockIdx.y * 4 * epn;
@@ -304,60 +430,57 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   }
   __syncthreads();
 
-  if (writer) {
-    if (blockIdx.y == 0)
-      for (int i = tid; i < R * epn; i += NT) a.etc[i] = s_etc[i];
-    if (tid == 0) {
-      a.remote_stats[2 * blockIdx.y] = s_nrem[rank];
-      a.remote_stats[2 * blockIdx.y + 1] = s_stat1[rank];
-    }
-  }
-
   // ---- my slice of the rank's entries -------------------------------------
-  int* dst = a.dst + (size_t)blockIdx.y * N;
-  int e = -1;
-  if (tid < n) {
-    e = topk[e0 + tid];
-    if ((unsigned)e >= (unsigned)E) e = -1;  // invalid id: becomes an entry that nobody copies
-  }
-  // lanes of my wave holding the same expert: one ballot per key bit
-  int pos = 0;
-  {
-    uint64_t same = __ballot(e >= 0);
-    const int nbits = 32 - __clz(E - 1 > 0 ? E - 1 : 1);
-    for (int b = 0; b < nbits; ++b) {
-      const bool bit = (e >> b) & 1;
-      const uint64_t bb = __ballot(bit);
-      same &= bit ? bb : ~bb;
-    }
-    if (e >= 0) {
-      pos = __popcll(same & mep_lanes_lt());
-      if (pos == 0)
-        atomicAdd(&s_wcnt[e * W4 + (wave >> 2)], __popcll(same) << (8 * (wave & 3)));
-    }
-  }
-  __syncthreads();
   // An entry with an invalid expert id gets destination rank R: dispatch and
   // combine skip such entries (they never write or read outside the R shards),
   // the duplicate-group builder matches no rank to it.
+  int* dst = a.dst + (size_t)blockIdx.y * N;
   int dv = R * NvS, dest = -1;  // fits: the host requires R*NvS <= INT32_MAX
   if (e >= 0) {
-    dest = 0;
-    int before = 0;
-    for (int w4 = 0; w4 <= (wave >> 2); ++w4) {
-      const unsigned word = (unsigned)s_wcnt[e * W4 + w4];
-      for (int b = 0; b < 4; ++b)
-        if (w4 * 4 + b < wave) before += (word >> (8 * b)) & 0xffu;
-    }
+    // entries of my expert in the waves before mine: one byte per wave, W4 words
+    // per expert; with my position in my own wave, my number within the slice
+    unsigned words[W4];
+#pragma unroll
+    for (int w4 = 0; w4 < W4; ++w4) words[w4] = (unsigned)s_wcnt[e * W4 + w4];
     // entries of expert e are numbered over (source rank, flat index) and cut
     // into the destinations' allocations in rank order
-    int g = s_prev[e] + s_hist[e] + before + pos;
-    if ((R & 3) == 0) {
-      const int4* row = (const int4*)(alloc + e * R);  // 16-byte aligned: tables start aligned, R % 4 == 0
+    int g = s_prev[e] + s_hist[e] + pos;
+    int4 c4[4];
+    const bool small_row = (R & 3) == 0 && R <= 16;
+    const int4* row = (const int4*)(alloc + e * R);  // 16-byte aligned when R % 4 == 0: tables start aligned
+    if (small_row) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        if (q4 * 4 < R) c4[q4] = row[q4];
+    }
+#pragma unroll
+    for (int w4 = 0; w4 < W4; ++w4) {
+      const int m = wave - 4 * w4;  // bytes of this word that belong to earlier waves
+      const unsigned mask = m >= 4 ? 0xffffffffu : (m <= 0 ? 0u : (1u << (8 * m)) - 1u);
+      g = (int)__builtin_amdgcn_sad_u8(words[w4] & mask, 0u, (unsigned)g);
+    }
+    if (small_row) {
+      // whole row read at once, then a search without branches
       bool found = false;
+      dest = R - 1;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4)
+        if (q4 * 4 < R) {
+          const int cs[4] = {c4[q4].x, c4[q4].y, c4[q4].z, c4[q4].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const bool hit = !found && (g < cs[j] || q4 * 4 + j == R - 1);
+            dest = hit ? q4 * 4 + j : dest;
+            found = found || hit;
+            g = found ? g : g - cs[j];
+          }
+        }
+    } else if ((R & 3) == 0) {
+      bool found = false;
+      dest = 0;
       for (int d4 = 0; d4 < R && !found; d4 += 4) {
-        const int4 c4 = row[d4 >> 2];
-        const int cs[4] = {c4.x, c4.y, c4.z, c4.w};
+        const int4 r4 = row[d4 >> 2];
+        const int cs[4] = {r4.x, r4.y, r4.z, r4.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           if (!found) {
@@ -366,7 +489,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
           }
       }
     } else {
-      for (; dest < R - 1; ++dest) {
+      for (dest = 0; dest < R - 1; ++dest) {
         const int c = alloc[e * R + dest];
         if (g < c) break;
         g -= c;
@@ -374,13 +497,31 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
     }
     dv = base[e * R + dest] + g;
   }
-  s_cd[tid] = dest;
-  __syncthreads();
-  if (tid < n) {
+  // a later entry of a token on a destination rank that an earlier entry of the
+  // token already has is a duplicate: stored as -dv - 1
+  bool dup = false;
+  if (16 % K == 0) {
+    // the K entries of a token sit in one DPP row: compare along the row
+    const int k = tid & (K - 1);
+#define MEP_DUP_STEP(J)                                                                      \
+  if (J < K) {                                                                               \
+    const int pj = __builtin_amdgcn_update_dpp(-2, dest, 0x110 + J, 0xf, 0xf, false);        \
+    dup |= J <= k && dest >= 0 && pj == dest;                                                \
+  }
+    MEP_DUP_STEP(1) MEP_DUP_STEP(2) MEP_DUP_STEP(3) MEP_DUP_STEP(4) MEP_DUP_STEP(5)
+    MEP_DUP_STEP(6) MEP_DUP_STEP(7) MEP_DUP_STEP(8) MEP_DUP_STEP(9) MEP_DUP_STEP(10)
+    MEP_DUP_STEP(11) MEP_DUP_STEP(12) MEP_DUP_STEP(13) MEP_DUP_STEP(14) MEP_DUP_STEP(15)
+#undef MEP_DUP_STEP
+  } else {
+    s_cd[tid] = dest;
+    __syncthreads();
     const int k = tid % K;
-    bool dup = false;
     for (int j = tid - k; j < tid; ++j) dup |= (dest >= 0 && s_cd[j] == dest);
-    dst[e0 + tid] = dup ? -dv - 1 : dv;
+  }
+  if (tid < n) dst[e0 + tid] = dup ? -dv - 1 : dv;
+  if (writer && tid == 0) {
+    a.remote_stats[2 * blockIdx.y] = s_nrem[rank];
+    a.remote_stats[2 * blockIdx.y + 1] = s_stat1[rank];
   }
 }
 
@@ -467,22 +608,24 @@ int plan_launch(const int32_t* tpe_RE, const int32_t* topk_nSK, int rank0, int n
   // only delays the planner and evicts itself
   constexpr size_t kWarmMax = (size_t)128 << 20;
   a.warm_vecs = warm ? (warm_bytes < kWarmMax ? warm_bytes : kWarmMax) / 16 : 0;
-  // one pass of eight loads per thread covers the range; at most ~two workgroups per CU
+  // eight loads per thread and pass; 1024 threads of warming per CU that the
+  // planning workgroups leave free (more gains nothing: 224 or 448 workgroups of
+  // 1024 threads read 59 MB in the same 10.7 us)
   int warm_groups = 0;
   if (a.warm_vecs) {
     const size_t per_wg = (size_t)c.nt * 8;
     const size_t want = (a.warm_vecs + per_wg - 1) / per_wg;
-    // what the CUs hold beside the planning workgroups at 2048 threads per CU
-    // (480 workgroups of 1024 threads on 256 CUs)
     const int cus = mep_device_cu_count();
     if (cus <= 0) return MEP_ERR_INVALID_ARG;
-    const int64_t room = (int64_t)cus * (2048 / c.nt) - (int64_t)c.groups * nranks;
+    const int64_t room = ((int64_t)cus - ((int64_t)c.groups * nranks * c.nt + 1023) / 1024) * (1024 / c.nt);
     const size_t cap = room > 0 ? (size_t)room : 0;
     warm_groups = (int)(want < cap ? want : cap);
   }
   dim3 grid(c.groups + warm_groups, nranks);
   hipStream_t st = (hipStream_t)stream;
-  if (c.nt == 1024) {
+  if (c.nt == 1024 && R == 8 && K == 8) {
+    hipLaunchKernelGGL((plan_kernel<1024, true, 8, 8>), grid, dim3(1024), c.lds_bytes, st, a);
+  } else if (c.nt == 1024) {
     hipLaunchKernelGGL((plan_kernel<1024, true>), grid, dim3(1024), c.lds_bytes, st, a);
   } else if (c.lds_tables) {
     hipLaunchKernelGGL((plan_kernel<256, true>), grid, dim3(256), c.lds_bytes, st, a);
