@@ -39,9 +39,9 @@ template <int NT>
 struct PlanLds {
   static constexpr int NW = NT / MEP_WAVE;
   static constexpr int W4 = (NW + 3) / 4;  // packed per-wave byte counters per expert
-  static constexpr int E_ARRAYS = 5 + W4;
+  static constexpr int E_ARRAYS = 6 + W4;
   static constexpr int R_ARRAYS = 6;
-  static constexpr int FIXED = 2 * NT;
+  static constexpr int FIXED = NT;
 };
 
 // RC, KC: the number of ranks and top-k as compile-time constants (0: taken
@@ -60,16 +60,16 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   int* s_prev = s_cnt + E;       // [E] tokens of the ranks before this one
   int* s_rem = s_prev + E;       // [E] not yet migrated
   int* s_etc = s_rem + E;        // [R*epn] remote experts per destination
-  int* s_hist = s_etc + E;       // [E] entries of this rank before my slice
-  int* s_wcnt = s_hist + E;      // [E*W4] per-wave counts, one byte per wave
+  int* s_hist = s_etc + E;       // [E] entries of this rank before my slice, or after it
+  int* s_own = s_hist + E;       // [E] tokens of this rank
+  int* s_wcnt = s_own + E;       // [E*W4] per-wave counts, one byte per wave
   int* s_gt = s_wcnt + W4 * E;   // [R] tokens per home group
   int* s_from = s_gt + R;        // [R] donor feeding this receiver (-1: none)
   int* s_quota = s_from + R;     // [R] tokens still to receive
   int* s_stat1 = s_quota + R;    // [R] slots elsewhere holding my experts
   int* s_nrem = s_stat1 + R;     // [R] remote experts on this destination
-  int* s_bal = s_nrem + R;       // [R]
-  int* s_ce = s_bal + R;         // [NT] expert of each entry of my slice
-  int* s_cd = s_ce + NT;         // [NT] destination rank of each entry
+  int* s_bal = s_nrem + R;       // [R] word 0: where counts of invalid expert ids go
+  int* s_cd = s_bal + R;         // [NT] destination rank of each entry
   int* tbl = kLdsTables ? (s_cd + NT)
                         : a.scratch + (size_t)(blockIdx.y * a.groups + blockIdx.x) * 2 * E * R;
   int* alloc = tbl;            // [E,R] tokens of expert e landing on rank d
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: roles branch on scalars
   if ((int)blockIdx.x >= a.groups) {
     // cache warmer: plain 16-byte loads, eight in flight.  The values only feed
     // a comparison that guards a sleep, so the loads stay and nothing is written.
@@ -117,9 +117,12 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) tv[j] = a.tpe[(j < R ? j : R - 1) * E + tid];
   }
-  // Per expert, this rank's entries that precede the workgroup's slice: needs
-  // nothing from the plan and is only used when the entries are resolved, so it
-  // runs beside the planning phases.  Wave 0 plans alone in the first of them
+  // Per expert, this rank's entries that precede the workgroup's slice - or
+  // those that follow it, where these are fewer: tokens_per_expert is the rank's
+  // count per expert (reference moonep/api.py:735), so what precedes is the
+  // total less the slice less what follows.  The count needs nothing from the
+  // plan and is only used when the entries are resolved, so it runs beside the
+  // planning phases.  Wave 0 plans alone in the first of them
   // (the serial greedy) while every other wave counts; in the two phases that
   // follow, waves 1..R plan (one per rank) and the waves above them count.  Each
   // part's first loads are issued one phase ahead.  With more ranks than that
@@ -130,9 +133,14 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   const bool count_a = wave >= 1, count_b = wave >= HWB;
   const bool hist_vec = (((uintptr_t)topk) & 15) == 0;
   const bool spread = R < HWB;
-  const int nv = hist_vec ? e0 >> 2 : 0;  // 16-byte vectors
-  const int hb1 = spread ? (int)(((int64_t)nv * 15) >> 5) : nv;
-  const int hb2 = spread ? (int)(((int64_t)nv * 24) >> 5) : nv;
+  const bool fwd = e0 <= N - (e0 + n);         // count what precedes the slice
+  const int c0 = fwd ? 0 : e0 + n, c1 = fwd ? e0 : N;
+  // entries [c0, c1) = a head up to a 16-byte boundary, vectors [v0, v1), a tail
+  const int v0 = (c0 + 3) >> 2;
+  const int v1 = hist_vec && (c1 >> 2) > v0 ? c1 >> 2 : v0;
+  const int head_end = min(4 * v0, c1), tail_start = max(4 * v1, head_end);
+  const int hb1 = v0 + (spread ? (int)(((int64_t)(v1 - v0) * 12) >> 5) : v1 - v0);
+  const int hb2 = v0 + (spread ? (int)(((int64_t)(v1 - v0) * 22) >> 5) : v1 - v0);
   const int4* t4 = (const int4*)topk;
   // loads v[u] = vector (b + t + u*nt) for those below `end`
   auto hist_load = [&](auto& v, int b, int end, int t, int nt) {
@@ -164,7 +172,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
     }
   };
   int4 ha[4], hb[6], hc[6];
-  if (count_a) hist_load(ha, 0, hb1, ta, NA);
+  if (count_a) hist_load(ha, v0, hb1, ta, NA);
 
   for (int i = tid; i < R; i += NT) {
     s_gt[i] = 0; s_from[i] = -1; s_quota[i] = 0; s_stat1[i] = 0; s_nrem[i] = 0;
@@ -176,7 +184,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   // ---- counts per expert, per home group --------------------------------
   const int epn_shift = (epn & (epn - 1)) == 0 ? 31 - __clz(epn) : -1;
   for (int ee = tid; ee < E; ee += NT) {
-    int c = 0, p = 0;
+    int c = 0, p = 0, own = 0;
     for (int r0 = 0; r0 < R; r0 += 8) {  // eight independent loads in flight
       int v[8];
       if (ee == tid && r0 == 0) {
@@ -191,10 +199,11 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       for (int j = 0; j < 8; ++j) {
         const int x = r0 + j < R ? v[j] : 0;
         p += r0 + j < rank ? x : 0;
+        own += r0 + j == rank ? x : 0;
         c += x;
       }
     }
-    s_cnt[ee] = c; s_prev[ee] = p; s_rem[ee] = c;
+    s_cnt[ee] = c; s_prev[ee] = p; s_rem[ee] = c; s_own[ee] = own;
     const int home = epn_shift >= 0 ? ee >> epn_shift : ee / epn;
     for (int d = 0; d < R; ++d) alloc[ee * R + d] = (d == home) ? c : 0;
     atomicAdd(&s_gt[home], c);
@@ -285,9 +294,9 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   };
   if (count_a) {
     rank_in_wave();
-    hist_part(ha, 0, hb1, ta, NA);
-    for (int i = (nv << 2) + ta; i < e0; i += NA)  // what 16-byte loads do not reach
-      atomicAdd(bin(topk[i]), 1);
+    hist_part(ha, v0, hb1, ta, NA);
+    for (int i = c0 + ta; i < head_end; i += NA) atomicAdd(bin(topk[i]), 1);
+    for (int i = tail_start + ta; i < c1; i += NA) atomicAdd(bin(topk[i]), 1);
   }
   __syncthreads();
 
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   // (waves 1..R, so that wave 0 is free)
   if (wave == 0) rank_in_wave();
   if (count_b && spread) {
-    hist_load(hc, hb2, nv, tb, NB);
+    hist_load(hc, hb2, v1, tb, NB);
     hist_part(hb, hb1, hb2, tb, NB);
   }
   for (int h = (wave + NW - 1) % NW; h < R; h += NW) {
@@ -376,30 +385,27 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
   __syncthreads();
 
   // ---- layout of every destination: one wave per destination -------------
-  if (count_b && spread) hist_part(hc, hb2, nv, tb, NB);
+  if (count_b && spread) hist_part(hc, hb2, v1, tb, NB);
   const bool tp_pow2 = (tp & (tp - 1)) == 0;
   for (int d = (wave + NW - 1) % NW; d < R; d += NW) {
-    const int lo = d * epn, hi = lo + epn;
+    const int lo = d * epn;
+    // Whatever is on d from elsewhere comes from the one home group that feeds d
+    // (s_from): its experts with tokens allocated to d, in ascending order.
+    const int hs = s_from[d] * epn;  // negative: d receives nothing
+    const int cnt_own = lane < epn ? alloc[(lo + lane) * R + d] : 0;  // read early: used after the scan
     int nremote = 0;
-    for (int c0 = 0; c0 < E; c0 += 256) {
-      int av[4];  // four reads in flight
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int ex = c0 + u * 64 + lane;
-        av[u] = ex < E ? alloc[ex * R + d] : 0;
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int ex = c0 + u * 64 + lane;
-        const bool sel = ex < E && (ex < lo || ex >= hi) && av[u] > 0;
+    if (hs >= 0) {
+      for (int c0 = 0; c0 < epn; c0 += 64) {
+        const int ex = hs + c0 + lane;
+        const bool sel = c0 + lane < epn && alloc[ex * R + d] > 0;
         const uint64_t m = __ballot(sel);
         if (sel) {
           const int slot = nremote + __popcll(m & mep_lanes_lt());
           if (slot < epn) s_etc[lo + slot] = ex;
-          atomicAdd(&s_stat1[epn_shift >= 0 ? ex >> epn_shift : ex / epn], 1);
         }
         nremote += __popcll(m);
       }
+      if (lane == 0 && nremote) atomicAdd(&s_stat1[s_from[d]], nremote);
     }
     for (int b = nremote + lane; b < epn; b += 64) s_etc[lo + b] = -1;
     if (lane == 0) s_nrem[d] = nremote;
@@ -415,7 +421,8 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       int eid = -1, cnt = 0;
       if (g < epn) eid = lo + g;
       else if (g < 2 * epn) eid = s_etc[lo + g - epn];
-      if (eid >= 0) cnt = alloc[eid * R + d];
+      if (c == 0 && g < epn) cnt = cnt_own;
+      else if (eid >= 0) cnt = alloc[eid * R + d];
       const int padded = tp_pow2 ? (cnt + tp - 1) & ~(tp - 1) : ((cnt + tp - 1) / tp) * tp;
       const int incl = mep_wave_incl_scan(padded);
       const int start = running + incl - padded;
@@ -444,7 +451,8 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
     for (int w4 = 0; w4 < W4; ++w4) words[w4] = (unsigned)s_wcnt[e * W4 + w4];
     // entries of expert e are numbered over (source rank, flat index) and cut
     // into the destinations' allocations in rank order
-    int g = s_prev[e] + s_hist[e] + pos;
+    const int counted = s_hist[e], mine_all = s_own[e];
+    int g = s_prev[e] + pos;
     int4 c4[4];
     const bool small_row = (R & 3) == 0 && R <= 16;
     const int4* row = (const int4*)(alloc + e * R);  // 16-byte aligned when R % 4 == 0: tables start aligned
@@ -458,6 +466,14 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
       const int m = wave - 4 * w4;  // bytes of this word that belong to earlier waves
       const unsigned mask = m >= 4 ? 0xffffffffu : (m <= 0 ? 0u : (1u << (8 * m)) - 1u);
       g = (int)__builtin_amdgcn_sad_u8(words[w4] & mask, 0u, (unsigned)g);
+    }
+    if (fwd) {
+      g += counted;
+    } else {  // the rank's total less my slice less what follows it
+      unsigned in_slice = 0;
+#pragma unroll
+      for (int w4 = 0; w4 < W4; ++w4) in_slice = __builtin_amdgcn_sad_u8(words[w4], 0u, in_slice);
+      g += mine_all - (int)in_slice - counted;
     }
     if (small_row) {
       // whole row read at once, then a search without branches
@@ -528,7 +544,7 @@ __global__ __launch_bounds__(NT) void plan_kernel(PlanArgs a) {
 size_t plan_lds_bytes(int nt, int E, int R, bool lds_tables) {
   const int nw = nt / MEP_WAVE;
   const int w4 = (nw + 3) / 4;
-  size_t ints = (size_t)(5 + w4) * E + 6 * (size_t)R + 2 * (size_t)nt;
+  size_t ints = (size_t)(6 + w4) * E + 6 * (size_t)R + (size_t)nt;
   if (lds_tables) ints += 2 * (size_t)E * R;
   return ints * sizeof(int);
 }
