@@ -100,6 +100,15 @@ def test_planner_matches_oracle_at_headline_shapes(cuda, S, H, K, E, R, mv):
     (12, 70, 96, 5, 32, 1.0),     # more than 64 experts per rank
     (8, 8, 262144, 8, 128, 1.0),  # counts too large for packed (value, index) keys
     (8, 512, 512, 4, 16, 1.0),    # E = 4096: per-expert arrays beyond 64 KB of LDS
+    # several workgroups per rank whose slices start off 16-byte boundaries (the count of
+    # earlier or later entries then has a scalar head and tail), ranks whose rows start
+    # unaligned (S*K odd), the compile-time R=8/K=8 kernel beside the generic one
+    (4, 4, 1501, 3, 8, 1.0),      # 1023 entries per workgroup, odd S*K
+    (8, 4, 1203, 7, 16, 1.5),     # 1022 entries per workgroup, R=8 without K=8
+    (8, 8, 2100, 8, 32, 1.0),     # R=8 and K=8, 17 workgroups, the last one partial
+    (4, 8, 3000, 8, 64, 2.0),     # K=8 without R=8: counting beside planning in the generic kernel
+    (16, 4, 2050, 4, 16, 1.0),    # more ranks than leave counting waves free
+    (3, 40, 1300, 5, 8, 1.0),     # experts per rank neither a power of two nor below 33
 ])
 def test_planner_wide_groups_match_oracle(cuda, R, epn, S, K, tp, sigma):
     """Shapes outside the golden table (R > 8, large counts): the CPU oracle,
@@ -256,4 +265,38 @@ def test_invalid_expert_ids_become_entries_that_nobody_copies(cuda):
                 written[d * NvS + int(start): d * NvS + int(start) + int(n)] = True
     assert bool((shards.view(R * NvS, H)[~written] == -3.0).all())
     assert torch.equal(out.cpu().float(), hid.float() * valid.sum(1, keepdim=True).float())
+    buf.destroy()
+
+
+@pytest.mark.parametrize("S,K,E,R,tp,rank", [
+    (1400, 8, 32, 8, 16, 5),    # 11 workgroups: ids to ignore in slices counted forwards and backwards
+    (1301, 3, 12, 4, 8, 1),     # slices off 16-byte boundaries
+])
+def test_invalid_expert_ids_across_workgroups(cuda, S, K, E, R, tp, rank):
+    """Ids outside [0, E) spread over a rank's entries, several workgroups per rank:
+    a workgroup counts the entries before its slice or those after it, whichever
+    are fewer, and neither count may include such an id."""
+    topk = torch.stack([routing.popularity_biased(S, K, E, R, r, 1.0, seed=12) for r in range(R)])
+    g = torch.Generator().manual_seed(77)
+    bad = topk[rank].clone().reshape(-1)
+    hit = torch.randperm(bad.numel(), generator=g)[: bad.numel() // 40]
+    junk = torch.tensor([E, -1, E + 3, 1 << 24, -(1 << 30)], dtype=torch.int32)
+    bad[hit] = junk[torch.randint(0, junk.numel(), (hit.numel(),), generator=g)]
+    valid = (bad >= 0) & (bad < E)
+    tpe = routing.tokens_per_expert(topk, E)
+    tpe[rank] = torch.bincount(bad[valid].long(), minlength=E).to(torch.int32)
+    gp = po.plan_global(tpe.numpy(), S, K, tp)
+    NvS = gp.NvS
+    raw = np.full(S * K, R * NvS, dtype=np.int64)
+    vmask = valid.numpy()
+    raw[vmask] = po.raw_dst_for_rank(gp, bad.numpy()[vmask], rank)
+    want = po.canonicalize_dst(raw, K, NvS)
+    want[~vmask] = R * NvS
+    buf = Buffer(S, 16, K, E, R, token_padding=tp, rank=rank)
+    ctx = buf._require_ctx()
+    plan, cu = allocate_planning_outputs(ctx)
+    launch_planning(ctx, bad.contiguous().to(cuda), tpe.to(cuda), cu, plan)
+    torch.cuda.synchronize()
+    assert np.array_equal(plan.dst.cpu().numpy(), want.astype(np.int32))
+    assert np.array_equal(cu.cpu().numpy(), gp.cu_seqlens[rank])
     buf.destroy()
