@@ -106,7 +106,9 @@ def test_planner_matches_oracle_at_headline_shapes(cuda, S, H, K, E, R, mv):
     (4, 4, 1501, 3, 8, 1.0),      # 1023 entries per workgroup, odd S*K
     (8, 4, 1203, 7, 16, 1.5),     # 1022 entries per workgroup, R=8 without K=8
     (8, 8, 2100, 8, 32, 1.0),     # R=8 and K=8, 17 workgroups, the last one partial
-    (4, 8, 3000, 8, 64, 2.0),     # K=8 without R=8: counting beside planning in the generic kernel
+    (4, 8, 3000, 8, 64, 2.0),     # the compile-time R=4/K=8 kernel
+    (16, 4, 1100, 8, 16, 1.0),    # the compile-time R=16/K=8 kernel: more ranks than leave counting waves free
+    (4, 8, 2500, 4, 64, 2.0),     # K=4, R=4: counting beside planning in the generic kernel
     (16, 4, 2050, 4, 16, 1.0),    # more ranks than leave counting waves free
     (3, 40, 1300, 5, 8, 1.0),     # experts per rank neither a power of two nor below 33
 ])
