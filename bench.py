@@ -19,8 +19,9 @@ Sections (all by default; `--sections chain` is the headline alone):
   chain    config 1 as above and the CPU baseline (the scalar C restatement
            oracle/mep_oracle.c on the host, same inputs); always measured;
   extras   the chain bounded to 32 .. 256 compute units (`chain_on_limited_cus`: 32 is
-           the reference's default `num_sms`) and the chain with six rotating sets of
-           destination shards;
+           the reference's default `num_sms`), the chain with six rotating sets of
+           destination shards, and the reference's separate kernels for duplicate rows
+           (all-rank plan, duplicate-group builder, epilogue, prologue);
   sweep    the chain at maxvio 0 .. 4 on both shapes with the headline's steps and
            warm-ups, three timings per point, the fastest kept (`maxvio_sweep`), and
            the chain at the configuration of the reference's own figure;
@@ -372,6 +373,52 @@ def chain_on_rotating_shards(ch, steps, nsets=6):
            "shard_sets": nsets, "GB_per_shard_set": ch.ctx["hidden_buf"].numel() * 2 / 1e9}
     del ctxs
     torch.cuda.empty_cache()
+    return out
+
+
+def split_duplicate_flow(ch, iters):
+    """The reference's separate kernels for duplicate rows, on the headline configuration:
+    every rank planned in one launch (the all-rank `dst` the duplicate map is built from), the
+    duplicate-group builder (reference moonep/dispatch.py:502-681), dispatch of the primaries
+    alone + the epilogue that expands them on the destination (dispatch_epilogue.py:44-304), the
+    prologue that folds duplicates into their primaries + the primaries-only combine
+    (combine_prologue.py:41-484), beside the fused forms the chain uses.  The epilogue and the
+    prologue work on this rank's shard as all R ranks' rows would fill it; the groups come from
+    the real all-rank plan, the rows' contents do not matter to the timing.  Launches repeat on
+    the same rows, part of which the 256 MB last-level cache still holds."""
+    import torch
+
+    from moonep_amd.combine import launch_combine, launch_combine_prologue
+    from moonep_amd.dispatch import launch_build_dedup, launch_dispatch, launch_dispatch_epilogue
+    from moonep_amd.planning import launch_planning_all_ranks
+
+    ctx, dev = ch.ctx, ch.topk.device
+    topk_all = ch.topk_all.to(torch.int32).contiguous().to(dev)
+    ch.plan_fn()
+    dst_all = launch_planning_all_ranks(ctx, topk_all, ch.tpe)[0]
+    torch.cuda.synchronize()
+    assert torch.equal(dst_all[ch.rank], ch.plan.dst)
+    out = {"plan_all_ranks_us": time_launches(lambda: launch_planning_all_ranks(ctx, topk_all, ch.tpe), iters),
+           "build_dedup_us": time_launches(lambda: launch_build_dedup(ctx, dst_all, ch.plan), iters)}
+    torch.cuda.synchronize()
+    groups, dups = (int(x) for x in ch.plan.dup_counts.cpu())
+    row = ch.H * 2
+    own_dups = int((ch.plan.dst < 0).sum())
+    out.update({"duplicate_groups_on_this_rank": groups, "duplicate_rows_on_this_rank": dups,
+                "duplicate_entries_of_this_rank": own_dups})
+    us = time_launches(lambda: launch_dispatch(ctx, ch.hidden[0], ch.wk, ch.plan, build_dedup_map=False,
+                                               write_dups=False), iters)
+    out["dispatch_primaries_us"] = us
+    us = time_launches(lambda: launch_dispatch_epilogue(ctx, ch.plan), iters)
+    out["dispatch_epilogue_us"] = us
+    out["dispatch_epilogue_roofline"] = hbm_roofline("dispatch_epilogue_kernel", (groups + dups) * row, us)
+    us = time_launches(lambda: launch_combine_prologue(ctx, ch.plan), iters)
+    out["combine_prologue_us"] = us
+    out["combine_prologue_roofline"] = hbm_roofline("combine_prologue_kernel", (2 * groups + dups) * row, us)
+    out["combine_primaries_us"] = time_launches(
+        lambda: launch_combine(ctx, ch.out[0], ch.plan.dst, ch.out_w, mode="primaries"), iters)
+    ctx["hidden_buf"].zero_()
+    torch.cuda.synchronize()
     return out
 
 
@@ -785,6 +832,7 @@ def main():
     if "extras" in args.sections:
         line["chain_on_limited_cus"] = chain_on_limited_cus(ch, sub_steps)
         line["chain_on_rotating_shards"] = chain_on_rotating_shards(ch, args.steps)
+        line["split_duplicate_flow"] = split_duplicate_flow(ch, sub_steps)
     ch.destroy()
     torch.cuda.empty_cache()
     tail = {}          # short summary keys, appended last

@@ -213,8 +213,17 @@ struct DupArgs {
 // Workgroups of 4 waves by default; of 16 waves when the caller bounds the number of
 // compute units (one workgroup per CU then, so each CU still has enough rows in flight).
 constexpr int kDupBlockMax = 1024;
+constexpr int kDupCH = 2;  // 1-KiB pieces of a row per wave and work item
 
-__global__ __launch_bounds__(kDupBlockMax) void epilogue_kernel(DupArgs a) {
+// A work item is (group, piece of the row): kDupCH consecutive 1-KiB pieces (64 lanes x 16
+// bytes).  Consecutive waves take consecutive pieces of one group, the waves grid-stride
+// over the items (their number is only known on the device).  A wave reads the group's
+// row numbers once, one per lane, before it touches a row, so that no row access waits for
+// an index load.
+// PROLOGUE: primary <- bf16(fp32 sum of the primary and its duplicates, in list order);
+// otherwise: every duplicate row <- the primary.
+template <bool PROLOGUE>
+__global__ __launch_bounds__(kDupBlockMax) void dup_rows_kernel(DupArgs a) {
   const int lane = threadIdx.x & 63;
   const int wpb = blockDim.x >> 6;
   const int gw = blockIdx.x * wpb + (threadIdx.x >> 6);
@@ -223,62 +232,69 @@ __global__ __launch_bounds__(kDupBlockMax) void epilogue_kernel(DupArgs a) {
   if (ng > a.NvS) ng = a.NvS;
   const size_t row_bytes = (size_t)a.H * 2;
   const int nvec = a.H / 8;
-  for (int g = gw; g < ng; g += nw) {
+  const int parts = (nvec + kDupCH * 64 - 1) / (kDupCH * 64);
+  const int64_t items = (int64_t)ng * parts;
+  for (int64_t it = gw; it < items; it += nw) {
+    const int g = (int)(it / parts);
+    const int part = (int)(it - (int64_t)g * parts);
     const int p = a.dup_groups[3 * g], start = a.dup_groups[3 * g + 1], n = a.dup_groups[3 * g + 2];
     if ((unsigned)p >= (unsigned)a.NvS || start < 0 || n <= 0 || (int64_t)start + n > a.NvS) continue;
-    const char* src = (const char*)a.shard + (size_t)p * row_bytes;
-    for (int c0 = 0; c0 < nvec; c0 += 4 * 64) {
-      mep_u4 v[4];
+    const int c0 = part * kDupCH * 64 + lane;
+    bool ok[kDupCH];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int c = c0 + i * 64 + lane;
-        if (c < nvec) v[i] = mep_ld16(src + (size_t)c * 16);
-      }
-      for (int j = 0; j < n; ++j) {
-        const int lo = a.dup_loffs[start + j];
+    for (int i = 0; i < kDupCH; ++i) ok[i] = c0 + i * 64 < nvec;
+    char* prow = (char*)a.shard + (size_t)p * row_bytes + (size_t)c0 * 16;
+    mep_u4 v[kDupCH];
+#pragma unroll
+    for (int i = 0; i < kDupCH; ++i)
+      if (ok[i]) v[i] = mep_ld16(prow + (size_t)i * 1024);
+    float acc[kDupCH][8];
+    if (PROLOGUE) {
+#pragma unroll
+      for (int i = 0; i < kDupCH; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc[i][2 * q] = 0.0f + mep_bf16_lo(v[i][q]);
+          acc[i][2 * q + 1] = 0.0f + mep_bf16_hi(v[i][q]);
+        }
+    }
+    for (int j0 = 0; j0 < n; j0 += 64) {
+      const int nj = n - j0 < 64 ? n - j0 : 64;
+      const int mine = lane < nj ? a.dup_loffs[start + j0 + lane] : -1;
+      for (int j = 0; j < nj; ++j) {
+        const int lo = __builtin_amdgcn_readlane(mine, j);
         if ((unsigned)lo >= (unsigned)a.NvS) continue;
-        char* row = (char*)a.shard + (size_t)lo * row_bytes;
+        char* row = (char*)a.shard + (size_t)lo * row_bytes + (size_t)c0 * 16;
+        if (PROLOGUE) {
+          mep_u4 d[kDupCH];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int c = c0 + i * 64 + lane;
-          if (c < nvec) mep_st16(row + (size_t)c * 16, v[i]);
+          for (int i = 0; i < kDupCH; ++i)
+            if (ok[i]) d[i] = mep_ld16(row + (size_t)i * 1024);
+#pragma unroll
+          for (int i = 0; i < kDupCH; ++i)
+            if (ok[i]) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                acc[i][2 * q] += mep_bf16_lo(d[i][q]);
+                acc[i][2 * q + 1] += mep_bf16_hi(d[i][q]);
+              }
+            }
+        } else {
+#pragma unroll
+          for (int i = 0; i < kDupCH; ++i)
+            if (ok[i]) mep_st16(row + (size_t)i * 1024, v[i]);
         }
       }
     }
-  }
-}
-
-__global__ __launch_bounds__(kDupBlockMax) void prologue_kernel(DupArgs a) {
-  const int lane = threadIdx.x & 63;
-  const int wpb = blockDim.x >> 6;
-  const int gw = blockIdx.x * wpb + (threadIdx.x >> 6);
-  const int nw = gridDim.x * wpb;
-  int ng = a.dup_counts[0];
-  if (ng > a.NvS) ng = a.NvS;
-  const size_t row_bytes = (size_t)a.H * 2;
-  const int nvec = a.H / 8;
-  for (int g = gw; g < ng; g += nw) {
-    const int p = a.dup_groups[3 * g], start = a.dup_groups[3 * g + 1], n = a.dup_groups[3 * g + 2];
-    if ((unsigned)p >= (unsigned)a.NvS || start < 0 || n <= 0 || (int64_t)start + n > a.NvS) continue;
-    char* prow = (char*)a.shard + (size_t)p * row_bytes;
-    for (int c = lane; c < nvec; c += 64) {
-      float acc[8];
+    if (PROLOGUE) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-      mep_u4 v = mep_ld16(prow + (size_t)c * 16);
+      for (int i = 0; i < kDupCH; ++i)
+        if (ok[i]) {
+          mep_u4 o;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { acc[2 * i] += mep_bf16_lo(v[i]); acc[2 * i + 1] += mep_bf16_hi(v[i]); }
-      for (int j = 0; j < n; ++j) {
-        const int lo = a.dup_loffs[start + j];
-        if ((unsigned)lo >= (unsigned)a.NvS) continue;
-        v = mep_ld16((const char*)a.shard + (size_t)lo * row_bytes + (size_t)c * 16);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { acc[2 * i] += mep_bf16_lo(v[i]); acc[2 * i + 1] += mep_bf16_hi(v[i]); }
-      }
-      mep_u4 o;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = mep_pack_bf16(acc[2 * i], acc[2 * i + 1]);
-      mep_st16(prow + (size_t)c * 16, o);
+          for (int q = 0; q < 4; ++q) o[q] = mep_pack_bf16(acc[i][2 * q], acc[i][2 * q + 1]);
+          mep_st16(prow + (size_t)i * 1024, o);
+        }
     }
   }
 }
@@ -439,7 +455,7 @@ extern "C" int mep_dispatch_epilogue(void* shard, const int32_t* dup_groups,
   DupArgs a{(uint16_t*)shard, dup_groups, dup_loffs, dup_counts, NvS, H};
   dim3 grid, block;
   dup_launch_shape(NvS, max_cus, &grid, &block);
-  hipLaunchKernelGGL(epilogue_kernel, grid, block, 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(dup_rows_kernel<false>, grid, block, 0, (hipStream_t)stream, a);
   return mep_launch_status();
 }
 
@@ -453,6 +469,6 @@ extern "C" int mep_combine_prologue(void* shard, const int32_t* dup_groups,
   DupArgs a{(uint16_t*)shard, dup_groups, dup_loffs, dup_counts, NvS, H};
   dim3 grid, block;
   dup_launch_shape(NvS, max_cus, &grid, &block);
-  hipLaunchKernelGGL(prologue_kernel, grid, block, 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(dup_rows_kernel<true>, grid, block, 0, (hipStream_t)stream, a);
   return mep_launch_status();
 }
