@@ -101,84 +101,93 @@ __global__ __launch_bounds__(kBlock) void dispatch_kernel(DispatchArgs a) {
 // ---------------------------------------------------------------------------
 // duplicate groups of one destination rank from every source rank's dst
 // ---------------------------------------------------------------------------
-// pass 1: per (source rank, token): how many of its K entries land on `rank`
-// pass 2: exclusive scan of (#groups, #duplicates) over the R*S tokens
-// pass 3: emit groups in token order
+// pass 1: per workgroup of tokens: (#groups, #duplicates) that `rank` holds of them
+// pass 2: every workgroup adds up the sums of the workgroups before it, scans its own
+//         tokens and emits their groups in token order; the last one stores the totals
 struct DedupArgs {
   const int* dst;  // [R, S*K]
   int* dup_groups; int* dup_loffs; int* dup_counts;
-  int* tok_dups;   // [R*S]   duplicates of each token on `rank` (entries - 1, >= 0)
-  int* blk_sums;   // [2*nblk] per-block (#groups, #dups), then their exclusive scan
+  int* blk_sums;   // [2*nblk] per-workgroup (#groups, #dups)
   int rank, S, K, R, NvS, ntok, nblk;
+  int vec;         // rows of dst can be read as 16-byte vectors
 };
 
 constexpr int kDedupBlock = 256;
+
+// entries of token t that land on `rank`: raw / NvS == rank, as a range test
+__device__ __forceinline__ int dedup_entries_on_rank(const DedupArgs& a, int t) {
+  const int lo = a.rank * a.NvS, hi = lo + a.NvS;  // fits: the host requires R*NvS <= INT32_MAX
+  auto on = [&](int v) { const int raw = v < 0 ? -v - 1 : v; return (int)(raw >= lo && raw < hi); };
+  const int* d = a.dst + (size_t)t * a.K;
+  int c = 0;
+  if (a.vec) {
+    const int4* d4 = (const int4*)d;
+    for (int k = 0; k < a.K / 4; ++k) {
+      const int4 v = d4[k];
+      c += on(v.x) + on(v.y) + on(v.z) + on(v.w);
+    }
+  } else {
+    for (int k = 0; k < a.K; ++k) c += on(d[k]);
+  }
+  return c;
+}
+
+// (sum of g, sum of d) over the workgroup, in every thread
+__device__ __forceinline__ void dedup_block_sums(int g, int d, int* s_g, int* s_d, int& tg, int& td) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int gs = mep_wave_incl_scan(g), ds = mep_wave_incl_scan(d);
+  if (lane == 63) { s_g[wave] = gs; s_d[wave] = ds; }
+  __syncthreads();
+  tg = 0; td = 0;
+  for (int w = 0; w < kDedupBlock / 64; ++w) { tg += s_g[w]; td += s_d[w]; }
+  __syncthreads();
+}
 
 __global__ __launch_bounds__(kDedupBlock) void dedup_count_kernel(DedupArgs a) {
   __shared__ int s_g[kDedupBlock / 64], s_d[kDedupBlock / 64];
   const int t = blockIdx.x * kDedupBlock + threadIdx.x;
   int nd = 0;
   if (t < a.ntok) {
-    const int* d = a.dst + (size_t)t * a.K;
-    int c = 0;
-    for (int k = 0; k < a.K; ++k) {
-      const int v = d[k];
-      const int raw = v < 0 ? -v - 1 : v;
-      c += (raw / a.NvS == a.rank);
-    }
+    const int c = dedup_entries_on_rank(a, t);
     nd = c > 1 ? c - 1 : 0;
-    a.tok_dups[t] = nd;
   }
-  // block totals
-  int g = nd > 0 ? 1 : 0;
-  int gs = mep_wave_incl_scan(g), ds = mep_wave_incl_scan(nd);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (lane == 63) { s_g[wave] = gs; s_d[wave] = ds; }
-  __syncthreads();
+  int tg, td;
+  dedup_block_sums(nd > 0 ? 1 : 0, nd, s_g, s_d, tg, td);
   if (threadIdx.x == 0) {
-    int tg = 0, td = 0;
-    for (int w = 0; w < kDedupBlock / 64; ++w) { tg += s_g[w]; td += s_d[w]; }
     a.blk_sums[2 * blockIdx.x] = tg;
     a.blk_sums[2 * blockIdx.x + 1] = td;
   }
-}
-
-// single workgroup: exclusive scan of the per-block sums, totals to dup_counts
-__global__ __launch_bounds__(1024) void dedup_scan_kernel(DedupArgs a) {
-  __shared__ int s_wg[16], s_wd[16];
-  __shared__ int s_carry[2];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (threadIdx.x == 0) { s_carry[0] = 0; s_carry[1] = 0; }
-  __syncthreads();
-  for (int b0 = 0; b0 < a.nblk; b0 += 1024) {
-    const int b = b0 + threadIdx.x;
-    int g = 0, d = 0;
-    if (b < a.nblk) { g = a.blk_sums[2 * b]; d = a.blk_sums[2 * b + 1]; }
-    const int gi = mep_wave_incl_scan(g), di = mep_wave_incl_scan(d);
-    if (lane == 63) { s_wg[wave] = gi; s_wd[wave] = di; }
-    __syncthreads();
-    int og = s_carry[0], od = s_carry[1];
-    for (int w = 0; w < wave; ++w) { og += s_wg[w]; od += s_wd[w]; }
-    if (b < a.nblk) { a.blk_sums[2 * b] = og + gi - g; a.blk_sums[2 * b + 1] = od + di - d; }
-    __syncthreads();
-    if (threadIdx.x == 1023) { s_carry[0] = og + gi; s_carry[1] = od + di; }
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) { a.dup_counts[0] = s_carry[0]; a.dup_counts[1] = s_carry[1]; }
 }
 
 __global__ __launch_bounds__(kDedupBlock) void dedup_emit_kernel(DedupArgs a) {
   __shared__ int s_g[kDedupBlock / 64], s_d[kDedupBlock / 64];
   const int t = blockIdx.x * kDedupBlock + threadIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int nd = t < a.ntok ? a.tok_dups[t] : 0;
+  // what the workgroups before this one hold
+  int pg = 0, pd = 0;
+  for (int b = threadIdx.x; b < (int)blockIdx.x; b += kDedupBlock) {
+    pg += a.blk_sums[2 * b];
+    pd += a.blk_sums[2 * b + 1];
+  }
+  int og, od;
+  dedup_block_sums(pg, pd, s_g, s_d, og, od);
+  int nd = 0;
+  if (t < a.ntok) {
+    const int c = dedup_entries_on_rank(a, t);
+    nd = c > 1 ? c - 1 : 0;
+  }
   const int g = nd > 0 ? 1 : 0;
   const int gi = mep_wave_incl_scan(g), di = mep_wave_incl_scan(nd);
   if (lane == 63) { s_g[wave] = gi; s_d[wave] = di; }
   __syncthreads();
-  int og = a.blk_sums[2 * blockIdx.x], od = a.blk_sums[2 * blockIdx.x + 1];
-  for (int w = 0; w < wave; ++w) { og += s_g[w]; od += s_d[w]; }
+  int tg = og, td = od;  // totals up to and including this workgroup
+  for (int w = 0; w < kDedupBlock / 64; ++w) {
+    if (w < wave) { og += s_g[w]; od += s_d[w]; }
+    tg += s_g[w]; td += s_d[w];
+  }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) { a.dup_counts[0] = tg; a.dup_counts[1] = td; }
   if (nd > 0) {
+    const int lo = a.rank * a.NvS, hi = lo + a.NvS;
     const int gidx = og + gi - 1;
     int dpos = od + di - nd;
     const int* d = a.dst + (size_t)t * a.K;
@@ -186,9 +195,8 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_emit_kernel(DedupArgs a) {
     for (int k = 0; k < a.K; ++k) {
       const int v = d[k];
       const int raw = v < 0 ? -v - 1 : v;
-      const int dr = raw / a.NvS;
-      if (dr != a.rank) continue;
-      const int loff = raw - dr * a.NvS;
+      if (raw < lo || raw >= hi) continue;
+      const int loff = raw - lo;
       if (first) {
         a.dup_groups[3 * gidx] = loff;
         a.dup_groups[3 * gidx + 1] = dpos;
@@ -378,9 +386,9 @@ extern "C" size_t mep_dedup_scratch_bytes(int S, int R) {
 
 namespace {
 
-// Fixed scratch of mep_build_dedup_static: per-token duplicate counts and the
-// per-workgroup sums of the three builder kernels, for callers that cannot
-// allocate.  1 MiB covers S*R up to 260 000 tokens (the headline shape needs
+// Fixed scratch of mep_build_dedup_static: what mep_dedup_scratch_bytes asks for (one
+// word per token and the builder's per-workgroup sums; the kernels use the sums), for
+// callers that cannot allocate.  1 MiB covers S*R up to 260 000 tokens (the headline shape needs
 // 129 KiB).  Every GPU the library runs on holds its own copy at its own
 // address until the process ends; host code must never pass the array's name
 // to a kernel (on the host it is only a handle for the symbol lookup) but the
@@ -418,8 +426,8 @@ extern "C" int mep_build_dedup_static(const int32_t* dst_RN, int rank, int S, in
   void* p = nullptr;
   const int rc = static_scratch_ptr(&p);
   if (rc != MEP_OK) return rc;
-  // Nothing needs clearing: the three kernels write every word of the scratch
-  // they later read (tok_dups[0, S*R), blk_sums[0, 2*nblk)) within this call.
+  // Nothing needs clearing: the first kernel writes every word of the scratch that
+  // the second reads (blk_sums[0, 2*nblk)) within this call.
   return mep_build_dedup(dst_RN, rank, S, K, R, NvS, dup_groups, dup_loffs, dup_counts, p,
                          kStaticDedupBytes, stream);
 }
@@ -436,11 +444,10 @@ extern "C" int mep_build_dedup(const int32_t* dst_RN, int rank, int S, int K, in
   a.rank = rank; a.S = S; a.K = K; a.R = R; a.NvS = NvS;
   a.ntok = S * R;
   a.nblk = (a.ntok + kDedupBlock - 1) / kDedupBlock;
-  a.tok_dups = (int*)workspace;
-  a.blk_sums = a.tok_dups + a.ntok;
+  a.blk_sums = (int*)workspace;
+  a.vec = (K % 4 == 0) && ((uintptr_t)dst_RN % 16 == 0);
   hipStream_t st = (hipStream_t)stream;
   hipLaunchKernelGGL(dedup_count_kernel, dim3(a.nblk), dim3(kDedupBlock), 0, st, a);
-  hipLaunchKernelGGL(dedup_scan_kernel, dim3(1), dim3(1024), 0, st, a);
   hipLaunchKernelGGL(dedup_emit_kernel, dim3(a.nblk), dim3(kDedupBlock), 0, st, a);
   return mep_launch_status();
 }
