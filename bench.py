@@ -411,10 +411,12 @@ def split_duplicate_flow(ch, iters):
     out["dispatch_primaries_us"] = us
     us = time_launches(lambda: launch_dispatch_epilogue(ctx, ch.plan), iters)
     out["dispatch_epilogue_us"] = us
-    out["dispatch_epilogue_roofline"] = hbm_roofline("dispatch_epilogue_kernel", (groups + dups) * row, us)
+    out["dispatch_epilogue_roofline"] = hbm_roofline("dup_rows_kernel<false> (dispatch epilogue)", (groups + dups) * row, us,
+                                                     measured_traffic("dispatch_epilogue")[0])
     us = time_launches(lambda: launch_combine_prologue(ctx, ch.plan), iters)
     out["combine_prologue_us"] = us
-    out["combine_prologue_roofline"] = hbm_roofline("combine_prologue_kernel", (2 * groups + dups) * row, us)
+    out["combine_prologue_roofline"] = hbm_roofline("dup_rows_kernel<true> (combine prologue)", (2 * groups + dups) * row, us,
+                                                    measured_traffic("combine_prologue")[0])
     out["combine_primaries_us"] = time_launches(
         lambda: launch_combine(ctx, ch.out[0], ch.plan.dst, ch.out_w, mode="primaries"), iters)
     ctx["hidden_buf"].zero_()
