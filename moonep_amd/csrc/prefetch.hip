@@ -31,7 +31,11 @@ struct SlotTable {
     e = smem; list = e + R * epn; off = list + R * epn; cur = off + epn + 1;
     active = cur + epn; misc = active + epn;
   }
-  // all threads of the workgroup call this
+  // All threads of the workgroup call this.  ORDERED: every expert's slots in ascending
+  // order (the reduction adds them in that order); otherwise in any order (a copy to every
+  // slot does not care), which all threads fill in at once instead of one wave walking the
+  // table.
+  template <bool ORDERED>
   __device__ void build(const int* etc, int rank, int R, int epn) {
     const int n = R * epn;
     const int lo = rank * epn;
@@ -61,27 +65,38 @@ struct SlotTable {
       }
       if (lane == 0) misc[0] = na;
       mep_wave_sync();
-      // slots in ascending order per expert
-      const int nbits = 32 - __clz(epn > 1 ? epn - 1 : 1);
-      for (int c = 0; c < n; c += 64) {
-        const int le = c + lane < n ? e[c + lane] : -1;
-        uint64_t same = __ballot(le >= 0);
-        for (int b = 0; b < nbits; ++b) {
-          const bool bit = (le >> b) & 1;
-          const uint64_t bb = __ballot(bit);
-          same &= bit ? bb : ~bb;
+      if (ORDERED) {
+        // slots in ascending order per expert
+        const int nbits = 32 - __clz(epn > 1 ? epn - 1 : 1);
+        for (int c = 0; c < n; c += 64) {
+          const int le = c + lane < n ? e[c + lane] : -1;
+          uint64_t same = __ballot(le >= 0);
+          for (int b = 0; b < nbits; ++b) {
+            const bool bit = (le >> b) & 1;
+            const uint64_t bb = __ballot(bit);
+            same &= bit ? bb : ~bb;
+          }
+          int base = 0, pos = 0;
+          if (le >= 0) { base = cur[le]; pos = __popcll(same & mep_lanes_lt()); }
+          mep_wave_sync();
+          if (le >= 0) {
+            if (pos == 0) cur[le] = base + __popcll(same);
+            list[base + pos] = c + lane;
+          }
+          mep_wave_sync();
         }
-        int base = 0, pos = 0;
-        if (le >= 0) { base = cur[le]; pos = __popcll(same & mep_lanes_lt()); }
-        mep_wave_sync();
-        if (le >= 0) {
-          if (pos == 0) cur[le] = base + __popcll(same);
-          list[base + pos] = c + lane;
-        }
-        mep_wave_sync();
       }
     }
     __syncthreads();
+    if (!ORDERED) {
+      // entries as (rank << 16 | slot): the division is done here, once per slot
+      for (int i = threadIdx.x; i < n; i += blockDim.x)
+        if (e[i] >= 0) {
+          const int d = i / epn;
+          list[atomicAdd(&cur[e[i]], 1)] = (d << 16) | (i - d * epn);
+        }
+      __syncthreads();
+    }
   }
 };
 
@@ -159,6 +174,8 @@ struct PrefetchArgs {
 // One tile of the copy: which tensor, which local expert, where in its matrix.
 struct PrefetchTile {
   int ti, le, step;
+  int beg, end;  // the expert's slots in the table's list
+  int first;     // the first of them (rank << 16 | slot)
   int64_t off;   // of this thread's vector 0
   bool whole;
 };
@@ -171,7 +188,7 @@ __global__ __launch_bounds__(kBlock) void prefetch_kernel(PrefetchArgs a) {
   extern __shared__ int smem[];
   SlotTable t;
   t.carve(smem, a.R, a.epn);
-  t.build(a.etc, a.rank, a.R, a.epn);
+  t.build<false>(a.etc, a.rank, a.R, a.epn);
   const unsigned n_active = (unsigned)__builtin_amdgcn_readfirstlane(t.misc[0]);
   if (n_active == 0) return;
   unsigned total = 0;
@@ -183,6 +200,11 @@ __global__ __launch_bounds__(kBlock) void prefetch_kernel(PrefetchArgs a) {
     while (w >= per * n_active) { w -= per * n_active; per = (unsigned)a.st[++p.ti].tiles; }
     const unsigned ai = w / per, tile = w - ai * per;
     p.le = __builtin_amdgcn_readfirstlane(t.active[ai]);
+    // the slot list is looked up here, while the previous tile's loads are in flight, so that
+    // nothing stands between the arrival of a tile and its stores
+    p.beg = __builtin_amdgcn_readfirstlane(t.off[p.le]);
+    p.end = __builtin_amdgcn_readfirstlane(t.off[p.le + 1]);
+    p.first = __builtin_amdgcn_readfirstlane(t.list[p.beg]);
     p.off = a.st[p.ti].first(tile, &p.step);
     p.whole = a.st[p.ti].whole(tile);
     return p;
@@ -200,10 +222,9 @@ __global__ __launch_bounds__(kBlock) void prefetch_kernel(PrefetchArgs a) {
   };
   auto store = [&](const PrefetchTile& p, const mep_u4* v) {
     const int64_t bytes = a.st[p.ti].bytes;
-    const int beg = t.off[p.le], end = t.off[p.le + 1];
-    for (int sidx = beg; sidx < end; ++sidx) {
-      const int rb = t.list[sidx];
-      const int d = rb / a.epn, b = rb - d * a.epn;
+    for (int sidx = p.beg; sidx < p.end; ++sidx) {
+      const int rb = sidx == p.beg ? p.first : __builtin_amdgcn_readfirstlane(t.list[sidx]);
+      const int d = rb >> 16, b = rb & 0xffff;
       char* dst = a.pool[p.ti] + (int64_t)d * a.rank_stride[p.ti] + (int64_t)b * bytes + p.off;
       if (p.whole) {
 #pragma unroll
@@ -392,7 +413,7 @@ __global__ __launch_bounds__(kBlock) void grad_reduce_kernel(ReduceArgs a) {
     }
     if (lane == 0) occ[a.epn] = n;
   }
-  t.build(a.etc, a.rank, a.R, a.epn);  // ends with a workgroup barrier
+  t.build<true>(a.etc, a.rank, a.R, a.epn);  // ends with a workgroup barrier
   const int n_active = (a.flags & MEP_REDUCE_CLEAR_ONLY) ? 0 : t.misc[0];
   const int n_clear = (a.flags & MEP_REDUCE_NO_CLEAR) ? 0 : occ[a.epn];
   const bool clear_as_read = a.flags == 0;  // own slots holding own experts, zeroed by their reader

@@ -111,6 +111,8 @@ def test_planner_matches_oracle_at_headline_shapes(cuda, S, H, K, E, R, mv):
     (4, 8, 2500, 4, 64, 2.0),     # K=4, R=4: counting beside planning in the generic kernel
     (16, 4, 2050, 4, 16, 1.0),    # more ranks than leave counting waves free
     (3, 40, 1300, 5, 8, 1.0),     # experts per rank neither a power of two nor below 33
+    (2, 1200, 700, 4, 8, 1.0),    # 256-thread workgroups with tables in scratch and two ranks: one wave counts beside the planning phases
+    (2, 600, 900, 2, 4, 1.5),     # 256-thread workgroups with tables in LDS, two ranks
 ])
 def test_planner_wide_groups_match_oracle(cuda, R, epn, S, K, tp, sigma):
     """Shapes outside the golden table (R > 8, large counts): the CPU oracle,
