@@ -189,6 +189,58 @@ def test_planner_random_small_shapes_match_oracle(cuda):
     assert checked >= 80
 
 
+def test_planner_random_multi_workgroup_shapes_match_oracle(cuda):
+    """Seeded sweep of shapes with several workgroups per rank (2 to 24), through every kernel
+    variant (compile-time R with top-8, the generic one), with the awkward routings of the
+    small-shape sweep: duplicates inside a token, a few hot experts, identical routing on all
+    ranks, skewed popularity."""
+    rng = np.random.default_rng(77031)
+    checked = 0
+    for it in range(48):
+        R = int(rng.choice([2, 4, 8, 16]))
+        epn = int(rng.integers(1, 17))
+        K = int(rng.choice([1, 2, 3, 5, 8, 8]))
+        S = int(rng.integers(300, 3001))
+        tp = int(rng.choice([1, 8, 16, 128]))
+        E = R * epn
+        kind = it % 4
+        if kind == 0:
+            topk = rng.integers(0, E, (R, S, K))
+        elif kind == 1:
+            hot = rng.integers(0, E, (max(1, min(E, 3)),))
+            topk = hot[rng.integers(0, hot.size, (R, S, K))]
+        elif kind == 2:
+            topk = np.repeat(rng.integers(0, E, (1, S, K)), R, axis=0)
+        else:
+            p = np.exp(rng.normal(0.0, 1.5, E))
+            p /= p.sum()
+            if K <= E:   # distinct experts per token: Gumbel top-k
+                g = rng.gumbel(size=(R, S, E)) + np.log(p)
+                topk = np.argsort(-g, axis=2)[:, :, :K]
+            else:
+                topk = rng.choice(E, (R, S, K), p=p)
+        topk = np.ascontiguousarray(topk).astype(np.int32)
+        tpe = np.stack([np.bincount(topk[r].reshape(-1), minlength=E) for r in range(R)]).astype(np.int32)
+        try:
+            gp, plans, dst_all_ref = oracle_world_plan(topk, tpe, tp)
+        except AssertionError:
+            continue   # more remote experts than slots on some rank: the reference asserts too
+        buf = Buffer(S, 16, K, E, R, token_padding=tp, rank=0)
+        dst_all, cu, etc, zfr, stats = launch_planning_all_ranks(
+            buf._require_ctx(), torch.from_numpy(topk).to(cuda), torch.from_numpy(tpe).to(cuda))
+        torch.cuda.synchronize()
+        tag = f"iter {it}: R={R} epn={epn} S={S} K={K} tp={tp} kind={kind}"
+        assert np.array_equal(dst_all.cpu().numpy(), dst_all_ref), tag
+        assert np.array_equal(cu.cpu().numpy(), gp.cu_seqlens), tag
+        assert np.array_equal(etc.cpu().numpy(), gp.experts_to_copy), tag
+        assert np.array_equal(zfr.cpu().numpy(), gp.zero_fill), tag
+        assert np.array_equal(stats.cpu().numpy(), gp.remote_stats), tag
+        buf.destroy()
+        checked += 1
+    print(f"{checked} random multi-workgroup shapes checked", flush=True)
+    assert checked >= 30
+
+
 @pytest.mark.parametrize("S,K,E,R,tp,warm_elems", [
     (4096, 8, 256, 8, 128, 4096 * 7168),   # the headline shape with its token rows
     (40, 3, 8, 4, 8, 40 * 64),             # one warming workgroup, mostly clamped loads
