@@ -548,7 +548,9 @@ class Buffer:
                     world.rendezvous(rank)
                     tpe = world.tpe_table(rank)
                 launch_planning(ctx, topk.reshape(-1), tpe, cu_seqlens, plan, warm=hidden_sh)
-                world.dst_all[rank].copy_(plan.dst)
+                if world.host_threads:
+                    # the other ranks' threads build their duplicate groups from it
+                    world.dst_all[rank].copy_(plan.dst)
         launch_dispatch(ctx, hidden_sh, route_weights_sk, plan, build_dedup_map=False,
                         write_dups=True, pdl_trigger=self.enable_pdl)
         if sync:
