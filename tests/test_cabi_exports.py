@@ -78,6 +78,7 @@ def test_error_codes_for_unsupported_shapes_alignment_and_scratch():
     assert plan(E=2050, S=256, K=1, NvS=1024) == -3        # planner tables need caller scratch
     assert plan(E=2050, S=256, K=1, NvS=1024, scratch=A + 4, sbytes=1 << 30) == -4   # misaligned scratch
     assert plan(E=1 << 16, R=2, S=256, K=1, NvS=1024, scratch=A, sbytes=1 << 40) == -2  # beyond the LDS limit
+    assert plan(E=5816, R=8, S=256, K=1, NvS=1024, scratch=A, sbytes=1 << 40) == -2     # one step beyond it (E = 5808 fills the 160 KB)
     assert lib.mep_plan_warm(A, A, 0, 4, 2, 8, 2, 8, 64, A, A, A, A, A, None, 0, A + 4, 64, None) == -4  # misaligned warm range
     # dispatch / combine: misaligned rows, weights without slots, bad mode, ragged H
     assert lib.mep_dispatch(A + 2, None, A, A, A, 64, None, 0, 0, 4, 64, 2, 2, 4, 64, 8, 0, None) == -4

@@ -100,6 +100,7 @@ def test_planner_matches_oracle_at_headline_shapes(cuda, S, H, K, E, R, mv):
     (12, 70, 96, 5, 32, 1.0),     # more than 64 experts per rank
     (8, 8, 262144, 8, 128, 1.0),  # counts too large for packed (value, index) keys
     (8, 512, 512, 4, 16, 1.0),    # E = 4096: per-expert arrays beyond 64 KB of LDS
+    (8, 726, 600, 4, 16, 1.0),    # E = 5808: exactly the 160 KB of LDS a workgroup can have (5816 is refused)
     # several workgroups per rank whose slices start off 16-byte boundaries (the count of
     # earlier or later entries then has a scalar head and tail), ranks whose rows start
     # unaligned (S*K odd), the compile-time R=8/K=8 kernel beside the generic one
