@@ -20,8 +20,9 @@ Sections (all by default; `--sections chain` is the headline alone):
            oracle/mep_oracle.c on the host, same inputs); always measured;
   extras   the chain bounded to 32 .. 256 compute units (`chain_on_limited_cus`: 32 is
            the reference's default `num_sms`), the chain with six rotating sets of
-           destination shards, and the reference's separate kernels for duplicate rows
-           (all-rank plan, duplicate-group builder, epilogue, prologue);
+           destination shards, the reference's separate kernels for duplicate rows
+           (all-rank plan, duplicate-group builder, epilogue, prologue), and the chain
+           called eagerly through Buffer.dispatch / Buffer.combine (`buffer_api_eager`);
   sweep    the chain at maxvio 0 .. 4 on both shapes with the headline's steps and
            warm-ups, three timings per point, the fastest kept (`maxvio_sweep`), and
            the chain at the configuration of the reference's own figure;
@@ -374,6 +375,32 @@ def chain_on_rotating_shards(ch, steps, nsets=6):
     del ctxs
     torch.cuda.empty_cache()
     return out
+
+
+def buffer_api_eager(ch, steps):
+    """Buffer.dispatch + Buffer.combine called eagerly, as a training loop without graphs calls
+    them (fresh plan every step, zero-copy views): what the host needs to issue a step (Python,
+    argument checks, ctypes) and what a step takes on the GPU with the queue kept full."""
+    import torch
+
+    buf = ch.buf
+    wk, tk = ch.wk, ch.topk
+
+    def step(i):
+        rows, rw, _, plan = buf.dispatch(ch.hidden[i % len(ch.hidden)], wk, tk, ch.tpe, zero_copy=True)
+        return buf.combine(plan, rows, rw, zero_copy=True)
+
+    for i in range(5):
+        step(i)
+    torch.cuda.synchronize()
+    n = max(50, 5 * steps)
+    t0 = time.perf_counter()
+    for i in range(n):
+        step(i)
+    t1 = time.perf_counter()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    return {"steps": n, "host_issue_us_per_step": (t1 - t0) * 1e6 / n, "us_per_step": (t2 - t0) * 1e6 / n}
 
 
 def split_duplicate_flow(ch, iters):
@@ -835,6 +862,7 @@ def main():
         line["chain_on_limited_cus"] = chain_on_limited_cus(ch, sub_steps)
         line["chain_on_rotating_shards"] = chain_on_rotating_shards(ch, args.steps)
         line["split_duplicate_flow"] = split_duplicate_flow(ch, sub_steps)
+        line["buffer_api_eager"] = buffer_api_eager(ch, args.steps)
     ch.destroy()
     torch.cuda.empty_cache()
     tail = {}          # short summary keys, appended last
